@@ -125,6 +125,14 @@ class LLMEngine:
                 raise ValueError(f"unsupported quantization {cfg.quantization!r} (supported: fp8)")
         self.model = model
         self._cuda = model.device.type == "cuda"
+        if getattr(model, "state_slots", False):
+            # recurrent state is per sequence, not per token: a prefix-cache hit would
+            # skip the tokens that build it, and KV handed between workers lacks it
+            if cfg.enable_prefix_caching:
+                log.info("%s carries recurrent state: prefix caching is off", type(model).__name__)
+                cfg.enable_prefix_caching = False
+            if cfg.host_kv_blocks or cfg.kv_shared:
+                raise ValueError(f"{type(model).__name__}: the host KV tier and KV transfer need per-token state only")
         if model.device.type == "cuda" and not model.fp8:
             model.enable_fused_mlp()  # prefill MLPs on the fused SwiGLU GEMM (csrc/kernels/gemm256.hip)
         model.fold_norms()  # norm weights into the projections: large forwards skip the norm kernels
@@ -154,7 +162,7 @@ class LLMEngine:
             if n > 0:
                 self.host_tier = HostKVTier(self.runner.kv_cache, n)
         self.kv = KVManager(self.runner.num_blocks, cfg.block_size, cfg.enable_prefix_caching, self._emit_events,
-                            host_tier=self.host_tier)
+                            host_tier=self.host_tier, state_slots=self.runner.num_state_slots)
         self.scheduler = Scheduler(
             SchedulerConfig(max_num_seqs=cfg.max_num_seqs, max_num_batched_tokens=cfg.max_num_batched_tokens,
                             max_model_len=cfg.max_model_len, max_prefill_streak=cfg.max_prefill_streak,
@@ -276,6 +284,8 @@ class LLMEngine:
         identifies the image content for prefix caching (derived from the
         embeddings when omitted)."""
         rid = request_id or uuid.uuid4().hex
+        if (remote_prefill or remote_decode) and self.runner.stateful:
+            raise ValueError(f"{type(self.model).__name__}: disaggregated prefill would leave the recurrent state behind")
         remote_read_blocks = remote_read_blocks or int((remote_meta or {}).get("read_blocks", 0))
         if not params.ignore_eos:
             params.stop_token_ids = list(dict.fromkeys(list(params.stop_token_ids) + self.eos_token_ids))

@@ -9,6 +9,12 @@
 * decode growth, free/release (a request's `cache_priority` ranks its blocks
   in the eviction order: lowest priority first, then oldest release --
   reference reuse.rs PriorityKey);
+* state slots: for models that carry per-sequence recurrent state (a running
+  matrix, the tail of a short convolution) the manager also owns `state_slots`
+  slots of the model's state tensors; a request gets one with its first pages
+  and returns it with them, lowest free slot first.  Such state is not
+  per-token, so it cannot be served from the prefix cache: the engine turns
+  prefix caching off for these models;
 * with a pinned-host tier: one per-worker view of both tiers for the router
   (a hash is Stored while either tier holds it, Removed when neither does)
   and write-ahead demotion of the next blocks to be evicted.
@@ -35,7 +41,7 @@ class KVEvent:
 
 class KVManager:
     def __init__(self, num_blocks: int, block_size: int, enable_prefix_caching: bool = True,
-                 event_sink: Callable[[list[KVEvent]], None] | None = None, host_tier=None):
+                 event_sink: Callable[[list[KVEvent]], None] | None = None, host_tier=None, state_slots: int = 0):
         rt = _native.runtime()
         if rt is None:
             raise RuntimeError("dynamo_exp_amd._C_runtime is required (BlockPool)")
@@ -51,6 +57,10 @@ class KVManager:
         self.prefix_queries = 0
         self.prefix_hit_tokens = 0
         self.prefix_query_tokens = 0
+        if state_slots and enable_prefix_caching:
+            raise ValueError("recurrent state slots and prefix caching exclude each other")
+        self.state_slots = state_slots
+        self._free_state = list(range(state_slots - 1, -1, -1))  # popped from the end: lowest slot first
         self._tiers: dict[int, int] = {}  # seq hash -> tier bits (1 device, 2 host), host tier only
         # write-ahead demotion keeps this many upcoming evictions copied to the host
         self.write_ahead_blocks = max(8, num_blocks // 64)
@@ -64,6 +74,25 @@ class KVManager:
 
     def blocks_needed(self, n_tokens: int) -> int:
         return (n_tokens + self.block_size - 1) // self.block_size
+
+    # ------------------------------------------------------------- recurrent state slots
+    def num_free_state(self) -> int:
+        return len(self._free_state)
+
+    def _take_state(self, req: Request) -> bool:
+        """A state slot for `req` unless it holds one (or the model has no state)."""
+        if not self.state_slots or req.state_slot is not None:
+            return True
+        if not self._free_state:
+            return False
+        req.state_slot = self._free_state.pop()
+        return True
+
+    def _drop_state(self, req: Request) -> None:
+        if req.state_slot is not None:
+            self._free_state.append(req.state_slot)
+            self._free_state.sort(reverse=True)
+            req.state_slot = None
 
     # ------------------------------------------------------------- prompt
     def prefix_hit_tokens_for(self, prompt: list[int]) -> int:
@@ -101,8 +130,9 @@ class KVManager:
             if self.host is not None:
                 host_hits = self.host.match(sh[len(hits):max_hit_blocks])
         need = self.blocks_needed(P + reserve_tokens) - len(hits)
-        new = self._allocate(max(0, need))
+        new = self._allocate(max(0, need)) if self._take_state(req) else None
         if new is None:
+            self._drop_state(req)
             if hits:
                 self.pool.free(hits)
             if host_hits:
@@ -137,11 +167,16 @@ class KVManager:
 
     # ------------------------------------------------------------- decode growth
     def ensure_slots(self, req: Request, total_tokens: int) -> bool:
+        fresh = req.state_slot is None
+        if not self._take_state(req):
+            return False
         need = self.blocks_needed(total_tokens) - len(req.block_ids)
         if need <= 0:
             return True
         new = self._allocate(need)
         if new is None:
+            if fresh:
+                self._drop_state(req)
             return False
         req.block_ids.extend(new)
         return True
@@ -172,6 +207,7 @@ class KVManager:
         if req.block_ids:
             self.pool.free(req.block_ids, int(getattr(req.params, "cache_priority", 0) or 0))
             req.block_ids = []
+        self._drop_state(req)
         self._flush_events()
 
     def set_priority(self, seq_hashes: list[int], priority: int) -> int:

@@ -104,6 +104,11 @@ class ModelRunner:
             self.kv_cache = torch.zeros(shape, dtype=cfg.kv_dtype, device=self.device)
         if not self.unified:
             self.kv_caches = [(self.kv_cache[i, 0], self.kv_cache[i, 1]) for i in range(L)]
+        # per-sequence recurrent state (models with `state_slots`): one slot per live
+        # request, handed out by the KV manager (Request.state_slot)
+        self.stateful = bool(getattr(model, "state_slots", False))
+        self.num_state_slots = cfg.max_num_seqs if self.stateful else 0
+        self.state = model.alloc_state(self.num_state_slots) if self.stateful else None
         self.graphs: dict[int, tuple] = {}
         self.graphs_sharded: dict[int, object] = {}  # TP > 1: vocab-sharded sampler variant
         self._res_tok = self._res_lp = None  # multi-step decode result buffers
@@ -125,7 +130,7 @@ class ModelRunner:
     def _auto_blocks(self) -> int:
         mc = self.model.cfg
         if self.unified:
-            per_block = self.model.kv_bytes_per_block(self.cfg.block_size, self.model.dtype)
+            per_block = max(1, self.model.kv_bytes_per_block(self.cfg.block_size, self.model.dtype))
         else:
             per_block = (mc.num_hidden_layers * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim *
                          torch.empty((), dtype=self.cfg.kv_dtype).element_size())
@@ -135,6 +140,8 @@ class ModelRunner:
         budget = total * self.cfg.gpu_memory_utilization - (total - free)
         # activations / graphs / logits headroom
         budget -= 6 << 30
+        if getattr(self.model, "state_slots", False):
+            budget -= self.model.state_bytes_per_slot() * self.cfg.max_num_seqs
         # fp8 prefill dequant scratch (bf16 K + V, one layer at a time)
         if self.fp8_scratch_cap:
             budget -= self.fp8_scratch_cap * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim * 2
@@ -146,7 +153,8 @@ class ModelRunner:
     @property
     def kv_bytes(self) -> int:
         if self.unified:
-            return sum(t.numel() * t.element_size() for k, v in self.kv_caches for t in ((k,) if v is k else (k, v)))
+            seen = {t.data_ptr(): t for kv in self.kv_caches for t in kv if t.numel()}  # shared caches count once
+            return sum(t.numel() * t.element_size() for t in seen.values())
         return self.kv_cache.numel() * self.kv_cache.element_size()
 
     def block_bytes_per_layer(self) -> int:
@@ -261,7 +269,21 @@ class ModelRunner:
             block_size=self.block_size,
             max_ctx=max(ctx) if ctx else 0,
         )
+        if self.stateful:
+            meta.state = self.state
+            meta.state_slots = self._to_dev(self._state_slots(allr, len(allr)), torch.int32)
+            meta.seq_rows = self._to_dev(np.asarray(list(cu) + [cu[-1] + i + 1 for i in range(len(decode))],
+                                                    dtype=np.int32), torch.int32)
         return self._to_dev(np.asarray(ids, dtype=np.int64), torch.int64), meta
+
+    @staticmethod
+    def _state_slots(reqs: list[Request], B: int) -> np.ndarray:
+        out = np.full(B, -1, dtype=np.int32)
+        for i, r in enumerate(reqs):
+            if r.state_slot is None:
+                raise RuntimeError(f"{r.request_id}: no recurrent-state slot")
+            out[i] = r.state_slot
+        return out
 
     def _plan_fp8_scratch(self, meta, reqs, num_new, ctx, cu) -> None:
         """Packed (and, past the cap, sequence-grouped) dequant scratch of an
@@ -500,6 +522,9 @@ class ModelRunner:
             block_size=self.block_size,
             max_ctx=int(ctx.max()) if B else 0,
         )
+        if self.stateful:
+            meta.state = self.state
+            meta.state_slots = self._to_dev(self._state_slots(reqs, B), torch.int32)
         if self.is_gpu and not self.unified:
             meta.workspace = ops.decode_workspace(B, self.model.n_q, self.model.head_dim, meta.n_parts, self.device)
         ids_t = self._to_dev(ids, torch.int64)
@@ -532,7 +557,7 @@ class ModelRunner:
         # one pinned host staging buffer + one device buffer, sliced per field (single H2D per step)
         self._layout = [("ids", torch.int64, maxB), ("pos", torch.int64, maxB), ("slots", torch.int64, maxB),
                         ("seeds", torch.int64, maxB), ("offs", torch.int64, maxB), ("ctx", torch.int32, maxB),
-                        ("topk", torch.int32, maxB), ("bt", torch.int32, maxB * mb), ("temp", torch.float32, maxB),
+                        ("topk", torch.int32, maxB), ("sslot", torch.int32, maxB), ("bt", torch.int32, maxB * mb), ("temp", torch.float32, maxB),
                         ("topp", torch.float32, maxB), ("minp", torch.float32, maxB)]
         nbytes = 0
         self._offsets = {}
@@ -587,6 +612,9 @@ class ModelRunner:
             block_size=self.block_size,
             max_ctx=self.cfg.max_model_len,
         )
+        if self.stateful:
+            meta.state = self.state
+            meta.state_slots = dv["sslot"][:B]
         hidden = self.model.forward(dv["ids"][:B], meta, self.kv_caches)
         if not full:
             self.model.sample_sharded(hidden, dv["temp"][:B], dv["seeds"][:B], dv["offs"][:B],
@@ -609,6 +637,7 @@ class ModelRunner:
         # dummy inputs: ctx 1, slot -1 (no KV writes), block 0
         self._hv["ctx"].fill_(1)
         self._hv["slots"].fill_(-1)
+        self._hv["sslot"].fill_(-1)  # no state is read or written
         self._hv["temp"].fill_(0)
         self._dev_buf.copy_(self._host_buf)
         stream = torch.cuda.Stream(self.device)
@@ -705,6 +734,8 @@ class ModelRunner:
         hv["pos"][:gb].numpy()[:] = pos
         hv["slots"][:gb].numpy()[:] = slots
         hv["ctx"][:gb].numpy()[:] = ctx
+        if self.stateful:
+            hv["sslot"][:gb].numpy()[:] = self._state_slots(reqs, gb)
         bt = hv["bt"][:gb].numpy()
         bt[:B] = 0
         for i, r in enumerate(reqs):

@@ -86,6 +86,9 @@ class Request:
     output: list[int] = field(default_factory=list)
     logprobs: list[float] = field(default_factory=list)
     block_ids: list[int] = field(default_factory=list)
+    # models with per-sequence recurrent state: the request's slot of the state tensors
+    # (KVManager hands it out with the first pages and takes it back with them)
+    state_slot: int | None = None
     num_computed: int = 0  # tokens whose KV is in the cache
     num_prefix_hit: int = 0  # prompt tokens served from the prefix cache
     block_hashes: list[int] = field(default_factory=list)  # local hashes of registered blocks

@@ -177,6 +177,8 @@ class LayeredConfig:
         n = 2 * self.vocab_size * W + W
         if self.architecture == "Bolinex":
             return n + self._bolinex_params()
+        if self.architecture == "Nefivik":
+            return n + self._nefivik_params()
         for L in self.layers:
             m, t = L["mixer"], L["type"]
             H, d, dv = m["heads"], m["dim"], m["vdim"]
@@ -213,6 +215,28 @@ class LayeredConfig:
             n += 2 * W * side + (W if side else 0)
         return n
 
+    def _nefivik_params(self) -> int:
+        W = self.hidden_size
+        side = (self.token_side or {}).get("dim", 0)
+        n = self.vocab_size * side * len(self.layers)
+        for L in self.layers:
+            m = L["mixer"]
+            H, d = m["heads"], m["dim"]
+            n += 2 * W + W * W + W  # sandwich norms and the gate of the mixer's result
+            if L["type"] == "general_delta":
+                lo = int(m.get("decay_rank") or max(8, d // 4))
+                n += 6 * H * d * W + 3 * H * d + lo * (W + H * d)
+            else:
+                G, dv, taps = m["kv_heads"], m["vdim"], int(m.get("conv") or 0)
+                own = (G * d + G * dv) if m.get("kv_from") is None else 0
+                n += (H * d + own) * (W + taps) + H * (W + 1) + W * H * dv
+            mlp = L.get("mlp")
+            if mlp:
+                E = mlp["router"]["experts"]
+                n += 2 * W + W * W + W + E * 3 * W * mlp["expert"]["ff"] + E * W
+            n += 2 * W * side + (W if side else 0)
+        return n
+
     def to_dict(self) -> dict:
         return dataclasses.asdict(self)
 
@@ -244,7 +268,7 @@ class LayeredConfig:
 
 
 # config.json `architecture` values served by LayeredConfig
-LAYERED_ARCHITECTURES = ("Bekulix", "Bolinex")
+LAYERED_ARCHITECTURES = ("Bekulix", "Bolinex", "Nefivik")
 
 
 def _bekulix_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, window, chunk, vocab=32000, streams=4):
@@ -280,6 +304,36 @@ def _bolinex_preset(name, W, ff, n_layers, heads, kv_heads, d, window, experts=0
     return LayeredConfig(name=name, architecture="Bolinex", vocab_size=vocab, hidden_size=W, layers=layers,
                          rms_norm_eps=1e-5, token_side={"dim": side} if side else None, learned_positions=True,
                          max_position_embeddings=max_positions)
+
+
+def _nefivik_preset(name, W, n_layers, heads, kv_heads, d, window, experts, top, expert_ff, groups=(1, 1), side=0,
+                    vocab=32000, conv=4, rot_dims=None, attn_every=3, limit=7.0):
+    """A Nefivik stack at a real model's layer sizes: generalized-delta-rule
+    layers with every `attn_every`-th layer a windowed sigmoid-attention layer
+    (short convolutions, partial rotary positions, head gate); every second
+    attention layer reads the previous attention layer's keys and values; all
+    feed-forwards are routed experts."""
+    rot_dims = rot_dims or d // 2
+    delta = {"type": "general_delta", "mixer": {"heads": heads, "dim": d}}
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "conv": conv,
+            "mask": {"size": window},
+            "rot": {"base": 500000.0, "dims": rot_dims,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff, "limit": limit},
+           "router": {"experts": experts, "top": top, "groups": {"count": groups[0], "keep": groups[1]}}}
+    layers, src = [], None
+    for i in range(n_layers):
+        if (i + 1) % attn_every:
+            layers.append({**delta, "mixer": dict(delta["mixer"]), "mlp": dict(mlp)})
+            continue
+        mixer = dict(attn)
+        if src is not None:
+            mixer["kv_from"], src = src, None
+        else:
+            src = i
+        layers.append({"type": "attention", "mixer": mixer, "mlp": dict(mlp)})
+    return LayeredConfig(name=name, architecture="Nefivik", vocab_size=vocab, hidden_size=W, layers=layers,
+                         rms_norm_eps=1e-5, token_side={"dim": side} if side else None)
 
 
 # CLIP ViT-L/14 at 336 px, the LLaVA-1.5 vision tower; features from the
@@ -346,6 +400,14 @@ PRESETS["bolinex-tiny"] = _bolinex_preset("bolinex-tiny", 256, 512, 4, 4, 2, 64,
 PRESETS["bolinex-8b-shapes"] = _bolinex_preset("bolinex-8b-shapes", 4096, 14336, 8, 32, 8, 128, 1024, experts=16,
                                                top=2, expert_ff=3584, shared_ff=3584, groups=(4, 2), side=256,
                                                vocab=128256)
+
+
+PRESETS["nefivik-tiny"] = _nefivik_preset("nefivik-tiny", 192, 6, 3, 1, 32, 48, experts=8, top=2, expert_ff=64,
+                                          groups=(4, 2), side=16, vocab=512, conv=4, rot_dims=16, limit=3.0)
+# Llama-3-8B's layer sizes (width 4096, 32 x 128 heads, 8 KV heads), 9 layers; 16 experts of a quarter
+# of the dense width, 2 chosen
+PRESETS["nefivik-8b-shapes"] = _nefivik_preset("nefivik-8b-shapes", 4096, 9, 32, 8, 128, 1024, experts=16, top=2,
+                                               expert_ff=3584, groups=(4, 2), side=256, vocab=128256)
 
 
 def get_config(name_or_path: str) -> ModelConfig:

@@ -68,6 +68,13 @@ class AttnMeta:
     row_tiles: torch.Tensor | None = None  # [n, 2] int32: (first row, rows) tiles of the prompt-chunk rows
     block_size: int = 0
     max_ctx: int = 0  # longest context of the step known on the host (0: unknown)
+    # models with per-sequence recurrent state (`state_slots` on the class): the slot of
+    # every sequence of the step in the runner's state tensors (-1: a padding row of a
+    # graph bucket), the first row of every sequence (None: row i is sequence i, a decode
+    # step), and the state tensors themselves (one tuple per layer, model.alloc_state)
+    state_slots: torch.Tensor | None = None  # [n_seq] int32
+    seq_rows: torch.Tensor | None = None  # [n_seq + 1] int32
+    state: list | None = None
 
 
 class TPGroup:

@@ -30,12 +30,19 @@ def _bolinex():
     return BolinexForCausalLM
 
 
+def _nefivik():
+    from .nefivik import NefivikForCausalLM
+
+    return NefivikForCausalLM
+
+
 # architecture -> (class loader, activation dtypes the class has kernels for)
 MODEL_REGISTRY = {
     "LlamaForCausalLM": (_llama, ("bfloat16",)),
     "LlavaForConditionalGeneration": (_llama, ("bfloat16",)),
     "Bekulix": (_bekulix, ("bfloat16", "float32")),
     "Bolinex": (_bolinex, ("bfloat16", "float32")),
+    "Nefivik": (_nefivik, ("bfloat16", "float32")),
 }
 
 

@@ -24,7 +24,8 @@ import torch
 from .. import _native
 
 MASKS = {"causal": 0, "window": 1, "chunk": 2}
-ACTS = {"relu": 0, "silu": 1, "gelu_tanh": 2, "sigmoid": 3, "relu2": 4}
+ACTS = {"relu": 0, "silu": 1, "gelu_tanh": 2, "sigmoid": 3, "relu2": 4, "tanh": 5, "swiglu_clamp": 6}
+WEIGHTS = {"softmax": 0, "sigmoid": 1}
 NORMS = {None: 0, "rms": 1, "layer": 2}
 MAX_STREAMS = 8
 # row attention: aim for this many waves per launch, never split a row's keys
@@ -100,9 +101,13 @@ def gather_rows(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
 def residual_step(X: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tensor | None = None,
                   c: torch.Tensor | None = None, c_w: torch.Tensor | None = None, eps: float = 1e-6,
                   norm: str | None = None, norm_w: torch.Tensor | None = None, norm_b: torch.Tensor | None = None,
-                  out_dtype: torch.dtype = torch.bfloat16, want_cast: bool = False):
+                  out_dtype: torch.dtype = torch.bfloat16, want_cast: bool = False,
+                  c_gate: torch.Tensor | None = None, c_gate_b: torch.Tensor | None = None):
     """One step of a single fp32 residual X [T, W], in place:
         X <- X + a + b + c / sqrt(mean(c^2) + eps) * c_w        (each addend optional)
+    with c_gate [T, W] (a column section, of the activation dtype) c is first
+    multiplied by sigmoid(c_gate + c_gate_b), in fp32: a sublayer result gated
+    element by element before it is normed into the residual;
     then, returned as (normed, cast):
         normed = norm(X) in out_dtype: 'rms'  X / sqrt(mean(X^2) + eps) * norm_w,
                                        'layer' (X - mean) / sqrt(var + eps) * norm_w + norm_b, None: nothing;
@@ -116,9 +121,11 @@ def residual_step(X: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tenso
     if norm not in NORMS or (norm and norm_w is None) or (norm == "layer" and norm_b is None) or \
             (c is not None and c_w is None):
         raise ValueError("residual_step: bad norm / weights")
-    for t, n in ((c_w, "c_w"), (norm_w, "norm_w"), (norm_b, "norm_b")):
+    if c_gate is not None and c is None:
+        raise ValueError("residual_step: a gate needs the addend c")
+    for t, n in ((c_w, "c_w"), (norm_w, "norm_w"), (norm_b, "norm_b"), (c_gate_b, "c_gate_b")):
         _fp32_param(t, n)
-    for t in (a, b, c):
+    for t in (a, b, c, c_gate):
         if t is not None and (t.shape != X.shape or t.stride(-1) != 1 or t.dtype != out_dtype):
             raise TypeError("residual_step: addends [T, W] with contiguous rows, of the activation dtype")
     if not X.is_cuda:
@@ -127,6 +134,8 @@ def residual_step(X: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tenso
                 X += t.float()
         if c is not None:
             cf = c.float()
+            if c_gate is not None:
+                cf = cf * torch.sigmoid(c_gate.float() + (c_gate_b if c_gate_b is not None else 0.0))
             X += cf * torch.rsqrt((cf * cf).mean(-1, keepdim=True) + eps) * c_w
         h = None
         if norm == "rms":
@@ -140,7 +149,7 @@ def residual_step(X: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tenso
     xc = torch.empty((T, W), dtype=out_dtype, device=X.device) if want_cast else None
     _m().residual_step(X.data_ptr(), _ptr(a), a.stride(0) if a is not None else 0, _ptr(b),
                        b.stride(0) if b is not None else 0, _ptr(c), c.stride(0) if c is not None else 0, _ptr(c_w),
-                       float(eps), NORMS[norm], _ptr(norm_w), _ptr(norm_b), _ptr(h), _ptr(xc), T, W,
+                       _ptr(c_gate), c_gate.stride(0) if c_gate is not None else 0, _ptr(c_gate_b), float(eps), NORMS[norm], _ptr(norm_w), _ptr(norm_b), _ptr(h), _ptr(xc), T, W,
                        int(out_dtype == torch.float32), _stream())
     return h, xc
 
@@ -190,37 +199,41 @@ def _act(z: torch.Tensor, act: str) -> torch.Tensor:
         return torch.sigmoid(z)
     if act == "relu2":
         return torch.relu(z) ** 2
+    if act == "tanh":
+        return torch.tanh(z)
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
-def glu_act(gu: torch.Tensor, act: str = "relu") -> torch.Tensor:
-    """[T, 2F] = [gate | up] -> act(gate) * up, [T, F]."""
-    T, F2 = gu.shape
-    F = F2 // 2
-    if act not in ACTS:
-        raise ValueError(f"unknown activation {act!r}")
-    if not gu.is_cuda:
-        g, u = gu.float().split(F, dim=1)
-        return (_act(g, act) * u).to(gu.dtype)
-    return act_mul(gu[:, :F], gu[:, F:], act)
+def glu_act(gu: torch.Tensor, act: str = "relu", limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """[T, 2F] = [gate | up] -> act(gate) * up, [T, F] (act_mul on the two halves)."""
+    F = gu.shape[1] // 2
+    return act_mul(gu[:, :F], gu[:, F:], act, limit, alpha)
 
 
-def act_mul(gate: torch.Tensor, up: torch.Tensor | None = None, act: str = "silu") -> torch.Tensor:
+def act_mul(gate: torch.Tensor, up: torch.Tensor | None = None, act: str = "silu", limit: float = 0.0,
+            alpha: float = 1.0) -> torch.Tensor:
     """act(gate) * up, [T, F] (up None: the activation alone).  gate and up may
     be column sections of wider tensors (contiguous rows, any row stride), e.g.
-    a gate that is part of a fused projection's output."""
+    a gate that is part of a fused projection's output.
+    'swiglu_clamp' is the clamped gated unit: with g = min(gate, limit) and
+    u = clamp(up, -limit, limit) the result is g * sigmoid(alpha * g) * (u + 1)."""
     T, F = gate.shape
     if act not in ACTS:
         raise ValueError(f"unknown activation {act!r}")
     if gate.stride(1) != 1 or (up is not None and (up.shape != gate.shape or up.stride(1) != 1 or
                                                    up.dtype != gate.dtype)):
         raise ValueError("act_mul: [T, F] sections with contiguous rows and one dtype")
+    if act == "swiglu_clamp" and (up is None or not limit > 0):
+        raise ValueError("act_mul: the clamped gated unit needs `up` and a positive limit")
     if not gate.is_cuda:
+        if act == "swiglu_clamp":
+            g, u = gate.float().clamp(max=limit), up.float().clamp(-limit, limit)
+            return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate.dtype)
         o = _act(gate.float(), act)
         return (o * up.float() if up is not None else o).to(gate.dtype)
     out = torch.empty((T, F), dtype=gate.dtype, device=gate.device)
     _m().act_mul(out.data_ptr(), gate.data_ptr(), gate.stride(0), _ptr(up), up.stride(0) if up is not None else 0, T, F,
-                 F, ACTS[act], _f32(gate), _stream())
+                 F, ACTS[act], float(limit), float(alpha), _f32(gate), _stream())
     return out
 
 
@@ -322,7 +335,8 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
               seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
               group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
               out_f32: bool = False, tiles: torch.Tensor | None = None, n_tile_rows: int = 0, softcap: float = 0.0,
-              dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
+              dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None, weights: str = "softmax",
+              head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of one step's rows: the first n_tile_rows rows (prompt chunks,
     cut into `tiles` [n, 2] = first row, row count) on the matrix-core prefill
     kernel where it applies, all other rows (decode tokens; every row when it
@@ -331,8 +345,9 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     T = q.shape[0]
     if not tile_attention_ok(q, d, dv) or not scale > 0:  # the matrix-core kernels fold a positive scale
         return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
-                             mask, size, parts, out_f32, softcap, dist_bias)
+                             mask, size, parts, out_f32, softcap, dist_bias, weights, head_bias, head_gate)
     _check_score_terms(softcap, dist_bias, n_qh)
+    _check_weight_terms(weights, head_bias, head_gate, q, n_qh, maps)
     if tiles is None:
         n_tile_rows = 0
     if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous() or \
@@ -349,20 +364,23 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     out = torch.empty((T, n_qh, dv), dtype=odt, device=q.device)
     common = (block_tables.data_ptr(), block_tables.stride(0), block_size)
     heads = (n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale), MASKS[mask], int(size),
-             float(softcap), _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0)
+             float(softcap), _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0,
+             WEIGHTS[weights], _ptr(head_bias))
+    gs = head_gate.stride(0) if head_gate is not None else 0
     if n_tile_rows:
         if seq is None or tiles.dtype != torch.int32 or not tiles.is_contiguous():
             raise TypeError("attention: prompt-chunk rows need seq and int32 tiles")
         _m().tile_attention(out.data_ptr(), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
                             positions.data_ptr(), seq.data_ptr(), *common, tiles.data_ptr(), tiles.shape[0], *heads,
-                            int(out_f32), _stream())
+                            _ptr(head_gate), gs, int(out_f32), _stream())
     n_dec = T - n_tile_rows
     if n_dec:  # decode rows: the heads of a K/V group share one wave's key tiles
         r0 = n_tile_rows
         ws = torch.empty((n_dec, n_qh, parts, 2 + dv), dtype=torch.float32, device=q.device)
         _m().group_decode(out[r0:].data_ptr(), ws.data_ptr(), q[r0:].data_ptr(), q.stride(0), kc.data_ptr(),
                           vc.data_ptr(), positions[r0:].data_ptr(), _ptr(seq[r0:] if seq is not None else None),
-                          *common, n_dec, *heads, parts, int(out_f32), _stream())
+                          *common, n_dec, *heads, _ptr(head_gate[r0:]) if head_gate is not None else 0, gs, parts,
+                          int(out_f32), _stream())
     return out
 
 
@@ -376,20 +394,38 @@ def _check_score_terms(softcap: float, dist_bias, n_qh: int) -> None:
                 raise ValueError("dist_bias: one (r1, r2) pair per query vector")
 
 
+def _check_weight_terms(weights: str, head_bias, head_gate, q: torch.Tensor, n_qh: int, maps: int) -> None:
+    if weights not in WEIGHTS:
+        raise ValueError(f"unknown attention weights {weights!r}")
+    _fp32_param(head_bias, "head_bias")
+    if head_bias is not None and head_bias.numel() != n_qh:
+        raise ValueError("head_bias: one number per query vector")
+    if head_gate is not None and (head_gate.shape != (q.shape[0], n_qh // maps) or head_gate.stride(1) != 1 or
+                                  head_gate.dtype != q.dtype):
+        raise ValueError("head_gate: [T, heads] of q's dtype with contiguous rows")
+
+
 def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
                   seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
                   group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
                   out_f32: bool = False, softcap: float = 0.0,
-                  dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
-    """Softmax attention of T rows over their sequences' paged caches.
+                  dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None, weights: str = "softmax",
+                  head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention of T rows over their sequences' paged caches.
     q [T, >= n_qh * d] (n_qh = heads * maps query vectors per row); returns
     [T, n_qh, dv].  Query vector qh reads K head (qh // maps // group) * maps +
     qh % maps and V head qh // maps // group.  The score of query position i
     and key position j is s = q . k * scale; with softcap > 0 then
     s <- softcap * tanh(s / softcap); with dist_bias = (r1, r2), fp32 [n_qh]
-    each, then s <- s - r1[qh] * ln(1 + r2[qh] * (i - j))."""
+    each, then s <- s - r1[qh] * ln(1 + r2[qh] * (i - j)); with head_bias
+    (fp32 [n_qh]) then s <- s + head_bias[qh].  weights 'softmax': the visible
+    keys' weights are softmax(s); 'sigmoid': every visible key weighs
+    sigmoid(s), not normalised over the keys.  With head_gate [T, heads]
+    (logits, a column section) head h's result is multiplied by
+    sigmoid(head_gate[:, h])."""
     T = q.shape[0]
     _check_score_terms(softcap, dist_bias, n_qh)
+    _check_weight_terms(weights, head_bias, head_gate, q, n_qh, maps)
     if mask not in MASKS:
         raise ValueError(f"unknown mask {mask!r}")
     if mask != "causal" and size < 1:
@@ -422,9 +458,14 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
             if dist_bias is not None:
                 dist = (p[:, None] - j[None, :]).clamp_min(0).float()
                 sc = sc - dist_bias[0][:, None, None] * torch.log1p(dist_bias[1][:, None, None] * dist[None])
+            if head_bias is not None:
+                sc = sc + head_bias[:, None, None]
             vis = (j[None, :] <= p[:, None]) & (j[None, :] >= first_visible(p, mask, size)[:, None])
             sc = sc.masked_fill(~vis[None], float("-inf"))
-            out[rows] = torch.einsum("hij,jhd->ihd", torch.softmax(sc, -1), V)
+            wt = torch.softmax(sc, -1) if weights == "softmax" else torch.sigmoid(sc)
+            out[rows] = torch.einsum("hij,jhd->ihd", wt, V)
+        if head_gate is not None:
+            out = out * torch.sigmoid(head_gate.float()).repeat_interleave(maps, 1)[:, :, None]
         return out.to(odt)
     if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous():
         raise TypeError("row_attention: caches contiguous and of q's dtype")
@@ -438,7 +479,9 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
     _m().row_attention(out.data_ptr(), _ptr(ws), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
                        positions.data_ptr(), _ptr(seq), block_tables.data_ptr(), block_tables.stride(0), block_size,
                        T, n_qh, maps, group, d, dv, Wk, Wv, float(scale), MASKS[mask], int(size), float(softcap),
-                       _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0, parts, _f32(q),
+                       _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0,
+                       WEIGHTS[weights], _ptr(head_bias), _ptr(head_gate),
+                       head_gate.stride(0) if head_gate is not None else 0, parts, _f32(q),
                        int(odt == torch.float32), _stream())
     return out
 

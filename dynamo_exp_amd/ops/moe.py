@@ -19,6 +19,8 @@ import torch
 from .. import _native
 from .mixers import _f32, _fp32_param, _ptr, _stream
 
+ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
+GROUP_SCORES = {"top2": 0, "max": 1}
 GLU_BLOCK = 32  # rows per gate / up block of weights interleaved for the fused SwiGLU epilogue
 
 
@@ -27,12 +29,13 @@ def _m():
 
 
 def route(z: torch.Tensor, correction: torch.Tensor | None, top: int, n_groups: int = 1, keep_groups: int = 1,
-          score: str = "sigmoid") -> tuple[torch.Tensor, torch.Tensor]:
+          score: str = "sigmoid", group_score: str = "top2") -> tuple[torch.Tensor, torch.Tensor]:
     """Expert choice per token from router logits z [T, E] (fp32).
-    s = sigmoid(z); the choice score is s + correction (correction None: s);
-    experts form n_groups equal groups of neighbours, a group's score is the
-    sum of its two largest choice scores (of its one score when groups hold a
-    single expert), and only experts of the keep_groups best groups compete;
+    s = sigmoid(z), or softmax(z) over all experts (`score`); the choice score
+    is s + correction (correction None: s); experts form n_groups equal groups
+    of neighbours, a group's score is the sum of its two largest choice scores
+    (of its one score when groups hold a single expert; group_score 'top2') or
+    its largest ('max'), and only experts of the keep_groups best groups compete;
     the `top` largest choice scores among those win.  Returns (idx [T, top]
     int32, w [T, top] fp32) with w = s of the chosen (no correction, not
     renormalised), best choice first; ties go to the lower index."""
@@ -40,17 +43,17 @@ def route(z: torch.Tensor, correction: torch.Tensor | None, top: int, n_groups: 
     if z.dtype != torch.float32 or not z.is_contiguous():
         raise TypeError("route: router logits are contiguous float32")
     _fp32_param(correction, "correction")
-    if score != "sigmoid":
-        raise ValueError(f"unknown router score {score!r}")
+    if score not in ROUTER_SCORES or group_score not in GROUP_SCORES:
+        raise ValueError(f"unknown router score {score!r} / group score {group_score!r}")
     if n_groups < 1 or E % n_groups or not 1 <= keep_groups <= n_groups or top < 1 or \
             top > keep_groups * (E // n_groups):
         raise ValueError("route: groups must divide the experts and hold at least `top` in those kept")
     if not z.is_cuda:
-        s = torch.sigmoid(z)
+        s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
         c = s + correction if correction is not None else s.clone()
         if n_groups > 1:
             per = E // n_groups
-            gs = c.view(T, n_groups, per).topk(min(2, per), -1).values.sum(-1)
+            gs = c.view(T, n_groups, per).topk(min(2 if group_score == "top2" else 1, per), -1).values.sum(-1)
             kept = torch.zeros(T, n_groups, dtype=torch.bool)
             kept.scatter_(1, gs.topk(keep_groups, -1).indices, True)
             c = c.masked_fill(~kept[:, :, None].expand(T, n_groups, per).reshape(T, E), float("-inf"))
@@ -59,7 +62,7 @@ def route(z: torch.Tensor, correction: torch.Tensor | None, top: int, n_groups: 
     idx = torch.empty((T, top), dtype=torch.int32, device=z.device)
     w = torch.empty((T, top), dtype=torch.float32, device=z.device)
     _m().moe_route(idx.data_ptr(), w.data_ptr(), z.data_ptr(), _ptr(correction), T, E, top, n_groups, keep_groups,
-                   _stream())
+                   ROUTER_SCORES[score], GROUP_SCORES[group_score], _stream())
     return idx, w
 
 
