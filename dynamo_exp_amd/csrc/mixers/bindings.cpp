@@ -19,13 +19,24 @@ int dxm_stream_step(float*, const void*, int64_t, const float*, const float*, co
 int dxm_embed_streams(float*, const void*, const int64_t*, int, int, int, int64_t, const void*, const int64_t*,
                       int64_t, int, hipStream_t);
 int dxm_gather_rows(void*, const void*, const int64_t*, int, int, int64_t, int, hipStream_t);
-int dxm_residual_step(float*, const void*, int64_t, const void*, int64_t, const void*, int64_t, const float*, float,
-                      int, const float*, const float*, void*, void*, int, int, int, hipStream_t);
-int dxm_act_mul(void*, const void*, int64_t, const void*, int64_t, int, int, int64_t, int, int, hipStream_t);
+int dxm_residual_step(float*, const void*, int64_t, const void*, int64_t, const void*, int64_t, const float*,
+                      const void*, int64_t, const float*, float, int, const float*, const float*, void*, void*, int, int,
+                      int, hipStream_t);
+int dxm_act_mul(void*, const void*, int64_t, const void*, int64_t, int, int, int64_t, int, float, float, int,
+                hipStream_t);
+int dxm_delta_rule(float*, float*, int, const void*, int64_t, const void*, int64_t, const void*, int64_t, const void*,
+                   int64_t, const void*, int64_t, const float*, const float*, float, float, const int64_t*, const int*,
+                   const int*, int, int, int, int, int, int, hipStream_t);
+int dxm_conv_rope_cache(void*, const void*, int64_t, const float*, int, const void*, int, const int64_t*,
+                        const int64_t*, const int*, const int*, const int*, int, int, int, int, int, int, const float*,
+                        int, void*, void*, int, hipStream_t);
+int dxm_conv_state_update(void*, int, const void*, int64_t, const int64_t*, const int*, const int*, int, int, int, int,
+                          int, hipStream_t);
+int dxm_head_norm_gate(void*, const float*, const float*, const void*, int64_t, int, int, int, float, int, hipStream_t);
 int dxm_headprep_cache(void*, int64_t, const int64_t*, const int64_t*, int, int, int, int, int, const float*,
                        const float*, float, float, double, void*, void*, int, int, int, const void*, int64_t, float,
                        int, hipStream_t);
-int dxm_moe_route(int*, float*, const float*, const float*, int, int, int, int, int, hipStream_t);
+int dxm_moe_route(int*, float*, const float*, const float*, int, int, int, int, int, int, int, hipStream_t);
 int dxm_moe_plan(int*, int*, const int*, int, int, hipStream_t);
 int dxm_grouped_gemm(void*, const void*, int64_t, const void*, const int*, const int*, int, int, int, int, int, int,
                      int, int, hipStream_t);
@@ -33,15 +44,15 @@ int dxm_moe_combine(void*, const void*, const float*, const void*, int64_t, int,
 int dxm_diff_combine(void*, const float*, int64_t, int, float, float, float, int, hipStream_t);
 int dxm_row_attention(void*, float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*,
                       const int*, int, int, int, int, int, int, int, int, int, int, float, int, int, float, const float*,
-                      const float*, int, int, int, hipStream_t);
+                      const float*, int, const float*, const void*, int64_t, int, int, int, hipStream_t);
 int dxm_tile_attention_ok(int, int);
 int dxm_tile_attention(void*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*,
                        int, int, const int*, int, int, int, int, int, int, int, int, float, int, int, float, const float*,
-                       const float*, int, hipStream_t);
+                       const float*, int, const float*, const void*, int64_t, int, hipStream_t);
 int dxm_group_decode(float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*, int,
                      int, int, int, int, int, int, int, int, int, float, int, int, float, const float*, const float*, int,
-                     hipStream_t);
-int dxm_merge_parts(void*, const float*, int64_t, int, int, int, hipStream_t);
+                     const float*, int, hipStream_t);
+int dxm_merge_parts(void*, const float*, int64_t, int, int, int, const void*, int64_t, int, int, int, hipStream_t);
 }
 
 static void check(int rc, const char* what) {
@@ -70,19 +81,49 @@ PYBIND11_MODULE(_C_mixers, m) {
     check(dxm_gather_rows(P(out), P(table), reinterpret_cast<const int64_t*>(ids), rows, W, vocab, f32, S(st)),
           "gather_rows");
   });
-  m.def("residual_step", [](u X, u a, int64_t as, u b, int64_t bs, u c, int64_t cs, u cw, float eps, int norm, u nw,
-                            u nb, u out, u xc, int rows, int W, int f32, u st) {
-    check(dxm_residual_step(F(X), P(a), as, P(b), bs, P(c), cs, F(cw), eps, norm, F(nw), F(nb), P(out), P(xc), rows, W,
-                            f32, S(st)),
+  m.def("residual_step", [](u X, u a, int64_t as, u b, int64_t bs, u c, int64_t cs, u cw, u cg, int64_t cgs, u cgb,
+                            float eps, int norm, u nw, u nb, u out, u xc, int rows, int W, int f32, u st) {
+    check(dxm_residual_step(F(X), P(a), as, P(b), bs, P(c), cs, F(cw), P(cg), cgs, F(cgb), eps, norm, F(nw), F(nb),
+                            P(out), P(xc), rows, W, f32, S(st)),
           "residual_step");
   });
-  m.def("act_mul", [](u out, u gate, int64_t gs, u up, int64_t us, int rows, int Fw, int64_t os, int act, int f32,
-                      u st) {
-    check(dxm_act_mul(P(out), P(gate), gs, P(up), us, rows, Fw, os, act, f32, S(st)), "act_mul");
+  m.def("act_mul", [](u out, u gate, int64_t gs, u up, int64_t us, int rows, int Fw, int64_t os, int act, float limit,
+                      float alpha, int f32, u st) {
+    check(dxm_act_mul(P(out), P(gate), gs, P(up), us, rows, Fw, os, act, limit, alpha, f32, S(st)), "act_mul");
   });
-  m.def("moe_route", [](u idx, u w, u z, u corr, int T, int E, int top, int n_groups, int keep, u st) {
-    check(dxm_moe_route(reinterpret_cast<int*>(idx), F(w), F(z), F(corr), T, E, top, n_groups, keep, S(st)),
+  m.def("moe_route", [](u idx, u w, u z, u corr, int T, int E, int top, int n_groups, int keep, int score,
+                        int group_max, u st) {
+    check(dxm_moe_route(reinterpret_cast<int*>(idx), F(w), F(z), F(corr), T, E, top, n_groups, keep, score, group_max,
+                        S(st)),
           "moe_route");
+  });
+  m.def("delta_rule", [](u out, u state, int n_slots, u r, int64_t rs, u k, int64_t ks, u v, int64_t vs, u a,
+                         int64_t as, u w, int64_t ws, u ab, u wb, float decay_scale, float key_eps, u pos, u seq_rows,
+                         u slots, int n_seq, int T, int H, int dk, int dv, int f32, u st) {
+    check(dxm_delta_rule(F(out), F(state), n_slots, P(r), rs, P(k), ks, P(v), vs, P(a), as, P(w), ws, F(ab), F(wb),
+                         decay_scale, key_eps, reinterpret_cast<const int64_t*>(pos),
+                         reinterpret_cast<const int*>(seq_rows), reinterpret_cast<const int*>(slots), n_seq, T, H, dk,
+                         dv, f32, S(st)),
+          "delta_rule");
+  });
+  m.def("conv_rope_cache", [](u q, u x, int64_t xs, u cw, int taps, u tail, int n_slots, u pos, u kv_slots, u row_seq,
+                              u seq_rows, u slots, int n_seq, int T, int n_q, int n_k, int d, int dv, u inv_freq,
+                              int half, u kc, u vc, int f32, u st) {
+    check(dxm_conv_rope_cache(P(q), P(x), xs, F(cw), taps, P(tail), n_slots, reinterpret_cast<const int64_t*>(pos),
+                              reinterpret_cast<const int64_t*>(kv_slots), reinterpret_cast<const int*>(row_seq),
+                              reinterpret_cast<const int*>(seq_rows), reinterpret_cast<const int*>(slots), n_seq, T,
+                              n_q, n_k, d, dv, F(inv_freq), half, P(kc), P(vc), f32, S(st)),
+          "conv_rope_cache");
+  });
+  m.def("conv_state_update", [](u tail, int n_slots, u x, int64_t xs, u pos, u seq_rows, u slots, int n_seq, int T,
+                                int C, int taps, int f32, u st) {
+    check(dxm_conv_state_update(P(tail), n_slots, P(x), xs, reinterpret_cast<const int64_t*>(pos),
+                                reinterpret_cast<const int*>(seq_rows), reinterpret_cast<const int*>(slots), n_seq, T,
+                                C, taps, f32, S(st)),
+          "conv_state_update");
+  });
+  m.def("head_norm_gate", [](u out, u o, u w, u gate, int64_t gs, int rows, int H, int dv, float eps, int f32, u st) {
+    check(dxm_head_norm_gate(P(out), F(o), F(w), P(gate), gs, rows, H, dv, eps, f32, S(st)), "head_norm_gate");
   });
   m.def("moe_plan", [](u order, u offsets, u idx, int R, int E, u st) {
     check(dxm_moe_plan(reinterpret_cast<int*>(order), reinterpret_cast<int*>(offsets),
@@ -112,29 +153,35 @@ PYBIND11_MODULE(_C_mixers, m) {
   m.def("tile_attention_ok", &dxm_tile_attention_ok);
   m.def("tile_attention", [](u out, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, u tiles,
                              int n_tiles, int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale,
-                             int mask, int size, float cap, u r1, u r2, int out_f32, u st) {
+                             int mask, int size, float cap, u r1, u r2, int wfn, u hbias, u gate, int64_t gs,
+                             int out_f32, u st) {
     check(dxm_tile_attention(P(out), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                              reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs,
                              reinterpret_cast<const int*>(tiles), n_tiles, n_qh, maps, group, d, dv, Wk, Wv, scale,
-                             mask, size, cap, F(r1), F(r2), out_f32, S(st)),
+                             mask, size, cap, F(r1), F(r2), wfn, F(hbias), P(gate), gs, out_f32, S(st)),
           "tile_attention");
   });
   m.def("group_decode", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                            int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                           int size, float cap, u r1, u r2, int parts, int out_f32, u st) {
+                           int size, float cap, u r1, u r2, int wfn, u hbias, u gate, int64_t gs, int parts,
+                           int out_f32, u st) {
     check(dxm_group_decode(F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                            reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
-                           maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), parts, S(st)),
+                           maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), wfn, F(hbias), parts,
+                           S(st)),
           "group_decode");
-    check(dxm_merge_parts(P(out), F(ws), (int64_t)rows * n_qh, parts, dv, out_f32, S(st)), "merge_parts");
+    check(dxm_merge_parts(P(out), F(ws), (int64_t)rows * n_qh, parts, dv, wfn, P(gate), gs, n_qh, maps, out_f32,
+                          S(st)),
+          "merge_parts");
   });
   m.def("row_attention", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                             int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                            int size, float cap, u r1, u r2, int parts, int f32, int out_f32, u st) {
+                            int size, float cap, u r1, u r2, int wfn, u hbias, u gate, int64_t gs, int parts, int f32,
+                            int out_f32, u st) {
     check(dxm_row_attention(P(out), F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                             reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
-                            maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), parts, f32, out_f32,
-                            S(st)),
+                            maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), wfn, F(hbias), P(gate), gs,
+                            parts, f32, out_f32, S(st)),
           "row_attention");
   });
 }

@@ -28,15 +28,17 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// One wave per token.  c[e] = sigmoid(z[e]) + corr[e] are the choice scores;
-// with n_groups > 1 only the experts of the `keep` groups with the largest
-// sum of their two best choice scores compete; the `top` best are written
-// with weight sigmoid(z) (no correction).
+// One wave per token.  c[e] = s[e] + corr[e] are the choice scores, s = sigmoid(z)
+// or softmax(z) over all experts; with n_groups > 1 only the experts of the `keep`
+// groups with the largest group score (the sum of their two best choice scores,
+// or with group_max their best) compete; the `top` best are written with weight
+// s (no correction).
 constexpr int kRouteWaves = 4;
 __global__ void __launch_bounds__(64 * kRouteWaves) moe_route_kernel(int* __restrict__ idx, float* __restrict__ w,
                                                                      const float* __restrict__ z,
                                                                      const float* __restrict__ corr, int T, int E,
-                                                                     int top, int n_groups, int keep) {
+                                                                     int top, int n_groups, int keep, int score,
+                                                                     int group_max) {
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t t = (int64_t)blockIdx.x * kRouteWaves + wv;
@@ -44,7 +46,18 @@ __global__ void __launch_bounds__(64 * kRouteWaves) moe_route_kernel(int* __rest
   float* c = sm + wv * (E + n_groups);
   float* gs = c + E;
   const float* zt = z + (on ? t : 0) * E;
-  for (int e = lane; e < E; e += 64) c[e] = 1.f / (1.f + expf(-zt[e])) + (corr ? corr[e] : 0.f);
+  // score 0: s = sigmoid(z); 1: s = softmax(z) over all experts (zmax, zinv: its maximum and 1 / sum)
+  float zmax = 0.f, zinv = 1.f;
+  if (score == 1) {
+    float mxv = -INFINITY;
+    for (int e = lane; e < E; e += 64) mxv = fmaxf(mxv, zt[e]);
+    zmax = wave_reduce_max(mxv);
+    float sm_ = 0.f;
+    for (int e = lane; e < E; e += 64) sm_ += expf(zt[e] - zmax);
+    zinv = 1.f / wave_reduce_sum(sm_);
+  }
+  for (int e = lane; e < E; e += 64)
+    c[e] = (score == 1 ? expf(zt[e] - zmax) * zinv : 1.f / (1.f + expf(-zt[e]))) + (corr ? corr[e] : 0.f);
   __syncthreads();
   if (n_groups > 1) {
     const int per = E / n_groups;
@@ -59,7 +72,7 @@ __global__ void __launch_bounds__(64 * kRouteWaves) moe_route_kernel(int* __rest
           b = v;
         }
       }
-      gs[g] = per > 1 ? a + b : a;
+      gs[g] = per > 1 && !group_max ? a + b : a;
     }
     __syncthreads();
     for (int k = 0; k < keep; ++k) {  // kept groups are marked +inf
@@ -98,7 +111,7 @@ __global__ void __launch_bounds__(64 * kRouteWaves) moe_route_kernel(int* __rest
       c[bi] = -INFINITY;
       if (on) {
         idx[t * top + k] = bi;
-        w[t * top + k] = 1.f / (1.f + expf(-zt[bi]));
+        w[t * top + k] = score == 1 ? expf(zt[bi] - zmax) * zinv : 1.f / (1.f + expf(-zt[bi]));
       }
     }
     __syncthreads();
@@ -354,15 +367,16 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(T* __restrict__ out, c
 extern "C" {
 
 int dxm_moe_route(int* idx, float* w, const float* z, const float* corr, int T, int E, int top, int n_groups,
-                  int keep, hipStream_t st) {
+                  int keep, int score, int group_max, hipStream_t st) {
   if (T <= 0) return 0;
+  if (score < 0 || score > 1) return 3;
   if (E < 1 || n_groups < 1 || E % n_groups || keep < 1 || keep > n_groups || top < 1 ||
       top > keep * (E / n_groups))
     return 1;
   const size_t lds = (size_t)kRouteWaves * (E + n_groups) * sizeof(float);
   if (lds > 48 * 1024) return 2;
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + kRouteWaves - 1) / kRouteWaves), dim3(64 * kRouteWaves), lds, st, idx,
-                     w, z, corr, T, E, top, n_groups, keep);
+                     w, z, corr, T, E, top, n_groups, keep, score, group_max);
   DX_CHECK_LAUNCH();
   return 0;
 }

@@ -1,0 +1,407 @@
+// Kernels with per-sequence state for gfx950: the generalized delta rule (a
+// running matrix per head), short causal convolutions over time fused with
+// rotary positions and the paged cache write, the convolution tail update, and
+// the per-head unit-RMS + gate that follows a recurrent mixer.
+//
+// State lives in slots ([slots, ...] tensors); a step names the slot of each of
+// its sequences (state_slots [n_seq], -1: a padding row that touches nothing)
+// and the first row of each (seq_rows [n_seq + 1]; null: row i is sequence i).
+// Rows of a sequence are consecutive positions.  A sequence whose first row of
+// the step is at position 0 starts from zero state, whatever its slot held.
+//
+// Every kernel is a template over the activation element (bf16 bits or float);
+// decays, removal rates, unit keys, the running matrix, angles and all sums are
+// fp32 whatever the element is.  Sizes are run-time arguments.
+#include "../kernels/common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+
+// ---------------------------------------------------------------------------
+// Generalized delta rule.  Per (sequence, head) a matrix S [dk, dv]:
+//     S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,   o_t = S_t^T r_t
+// with w_t = exp(-decay_scale * sigmoid(wl_t + w_bias)), a_t = sigmoid(al_t + a_bias),
+// u_t = k_t / sqrt(sum(k_t^2) + key_eps).  Columns of S are independent, so a
+// thread owns kRows consecutive rows of one column in registers, R threads
+// (neighbouring lanes) share a column and join their partial dot products by
+// lane exchanges, and a workgroup of 256 threads owns 256 / R columns of one
+// (sequence, head).  The state tensor is stored column-major per head
+// ([slots, H, dv, dk]) so that a wave's state traffic is one contiguous run.
+// Tokens are staged through LDS kTok at a time: raw r, k, a, w, v rows are
+// fetched into registers one block ahead (their latency hides behind the
+// current block's recurrence), committed, transformed in place (sums of
+// squares by wave reductions), and consumed token by token.
+constexpr int kRows = 16;  // state rows per thread
+constexpr int kTok = 8;    // tokens per staged block
+constexpr int kDThreads = 256;
+
+struct DeltaArgs {
+  float* out;    // [T, H * dv]
+  float* state;  // [slots, H, dv, dk]
+  const void *r, *k, *v, *a, *w;
+  int64_t rs, ks, vs, as, ws;  // row strides (elements)
+  const float* a_bias;         // [H * dk] or null
+  const float* w_bias;
+  float decay_scale, key_eps;
+  const int64_t* pos;
+  const int* seq_rows;  // null: row i is sequence i
+  const int* slots;
+  int n_slots, T, H, dk, dv;
+};
+
+template <typename T, int R>
+__global__ void __launch_bounds__(kDThreads) delta_rule_kernel(DeltaArgs g) {
+  constexpr int kCols = kDThreads / R;      // columns per workgroup
+  constexpr int kDkp = kRows * R;           // padded key width
+  constexpr int kE = (kTok * kDkp + kDThreads - 1) / kDThreads;   // staged elements per thread and array
+  constexpr int kEv = (kTok * kCols + kDThreads - 1) / kDThreads;
+  __shared__ __attribute__((aligned(16))) float sr[kTok][kDkp];
+  __shared__ __attribute__((aligned(16))) float sk[kTok][kDkp];
+  __shared__ __attribute__((aligned(16))) float su[kTok][kDkp];
+  __shared__ __attribute__((aligned(16))) float sw[kTok][kDkp];
+  __shared__ __attribute__((aligned(16))) float sa[kTok][kDkp];
+  __shared__ float sv[kTok][kCols];
+  const int tid = threadIdx.x, part = tid % R, c = tid / R;
+  const int s = blockIdx.x, h = blockIdx.y, j = blockIdx.z * kCols + c;
+  const int r0 = g.seq_rows ? g.seq_rows[s] : s;
+  const int r1 = g.seq_rows ? g.seq_rows[s + 1] : s + 1;
+  const int slot = g.slots[s];
+  const int n = r1 - r0;
+  if (n <= 0 || r0 < 0 || r1 > g.T) return;
+  const bool col_ok = j < g.dv;
+  if (slot < 0 || slot >= g.n_slots) {  // padding rows: a defined result, no state
+    if (col_ok && part == 0)
+      for (int t = r0; t < r1; ++t) g.out[(int64_t)t * g.H * g.dv + h * g.dv + j] = 0.f;
+    return;
+  }
+  const int i0 = part * kRows;
+  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv + (col_ok ? j : 0)) * g.dk + i0;
+  const bool fresh = g.pos[r0] == 0;
+  const bool vec = g.dk % 4 == 0 && i0 + kRows <= g.dk;
+  float S[kRows];
+#pragma unroll
+  for (int q = 0; q < kRows; ++q) S[q] = 0.f;
+  if (!fresh && col_ok) {
+    if (vec) {
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(sp + q);
+        S[q] = x[0], S[q + 1] = x[1], S[q + 2] = x[2], S[q + 3] = x[3];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < kRows; ++q)
+        if (i0 + q < g.dk) S[q] = sp[q];
+    }
+  }
+  const T* pr = (const T*)g.r + (int64_t)h * g.dk;
+  const T* pk = (const T*)g.k + (int64_t)h * g.dk;
+  const T* pa = (const T*)g.a + (int64_t)h * g.dk;
+  const T* pw = (const T*)g.w + (int64_t)h * g.dk;
+  const T* pv = (const T*)g.v + (int64_t)h * g.dv + blockIdx.z * kCols;
+  float fr[kE], fk[kE], fa[kE], fw[kE], fv[kEv];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int e = 0; e < kE; ++e) {
+      const int idx = tid + e * kDThreads, tt = idx / kDkp, ch = idx % kDkp;
+      const bool ok = idx < kTok * kDkp && t0 + tt < n && ch < g.dk;
+      const int64_t row = r0 + t0 + tt;
+      fr[e] = ok ? ldf<T>(pr, row * g.rs + ch) : 0.f;
+      fk[e] = ok ? ldf<T>(pk, row * g.ks + ch) : 0.f;
+      fa[e] = ok ? ldf<T>(pa, row * g.as + ch) : 0.f;
+      fw[e] = ok ? ldf<T>(pw, row * g.ws + ch) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < kEv; ++e) {
+      const int idx = tid + e * kDThreads, tt = idx / kCols, cc = idx % kCols;
+      const bool ok = idx < kTok * kCols && t0 + tt < n && blockIdx.z * kCols + cc < g.dv;
+      fv[e] = ok ? ldf<T>(pv, (int64_t)(r0 + t0 + tt) * g.vs + cc) : 0.f;
+    }
+  };
+  fetch(0);
+  const int lane = tid & 63, wv = tid >> 6;
+  for (int t0 = 0; t0 < n; t0 += kTok) {
+    __syncthreads();  // the previous block's tokens are consumed
+#pragma unroll
+    for (int e = 0; e < kE; ++e) {
+      const int idx = tid + e * kDThreads, tt = idx / kDkp, ch = idx % kDkp;
+      if (idx < kTok * kDkp) {
+        sr[tt][ch] = fr[e];
+        sk[tt][ch] = fk[e];
+        const bool in = ch < g.dk;
+        sa[tt][ch] = in ? sigmoidf_(fa[e] + (g.a_bias ? g.a_bias[h * g.dk + ch] : 0.f)) : 0.f;
+        sw[tt][ch] = in ? expf(-g.decay_scale * sigmoidf_(fw[e] + (g.w_bias ? g.w_bias[h * g.dk + ch] : 0.f))) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < kEv; ++e) {
+      const int idx = tid + e * kDThreads;
+      if (idx < kTok * kCols) sv[idx / kCols][idx % kCols] = fv[e];
+    }
+    __syncthreads();
+    if (t0 + kTok < n) fetch(t0 + kTok);
+    // unit keys: one wave per token, kTok / 4 tokens each
+    for (int tt = wv; tt < kTok; tt += kDThreads / 64) {
+      float ss = 0.f;
+      for (int ch = lane; ch < kDkp; ch += 64) ss += sk[tt][ch] * sk[tt][ch];
+      const float inv = rsqrtf(wave_reduce_sum(ss) + g.key_eps);
+      for (int ch = lane; ch < kDkp; ch += 64) {
+        const float u = sk[tt][ch] * inv;
+        su[tt][ch] = u;
+        sa[tt][ch] *= u;
+      }
+    }
+    __syncthreads();
+    const int nt = n - t0 < kTok ? n - t0 : kTok;
+    for (int tt = 0; tt < nt; ++tt) {
+      float u[kRows], x[kRows];
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(u + q) = *reinterpret_cast<const f32x4*>(&su[tt][i0 + q]);
+      float us = 0.f;
+#pragma unroll
+      for (int q = 0; q < kRows; ++q) us += u[q] * S[q];
+#pragma unroll
+      for (int o = 1; o < R; o <<= 1) us += __shfl_xor(us, o, 64);
+      const float vj = sv[tt][c];
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sw[tt][i0 + q]);
+#pragma unroll
+      for (int q = 0; q < kRows; ++q) S[q] *= x[q];
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sa[tt][i0 + q]);
+#pragma unroll
+      for (int q = 0; q < kRows; ++q) S[q] -= x[q] * us;
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sk[tt][i0 + q]);
+#pragma unroll
+      for (int q = 0; q < kRows; ++q) S[q] += x[q] * vj;
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sr[tt][i0 + q]);
+      float o_ = 0.f;
+#pragma unroll
+      for (int q = 0; q < kRows; ++q) o_ += x[q] * S[q];
+#pragma unroll
+      for (int o = 1; o < R; o <<= 1) o_ += __shfl_xor(o_, o, 64);
+      if (part == 0 && col_ok) g.out[(int64_t)(r0 + t0 + tt) * g.H * g.dv + h * g.dv + j] = o_;
+    }
+  }
+  if (col_ok) {
+    if (vec) {
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(sp + q) = f32x4{S[q], S[q + 1], S[q + 2], S[q + 3]};
+    } else {
+#pragma unroll
+      for (int q = 0; q < kRows; ++q)
+        if (i0 + q < g.dk) sp[q] = S[q];
+    }
+  }
+}
+
+template <typename T, int R>
+void launch_delta(const DeltaArgs& g, int n_seq, hipStream_t st) {
+  const int cols = kDThreads / R;
+  hipLaunchKernelGGL((delta_rule_kernel<T, R>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(kDThreads), 0, st, g);
+}
+
+// ---------------------------------------------------------------------------
+// Short causal convolution over time on the leading C = n_q d + n_k (d + dv)
+// columns of a fused projection, then rotary positions on the first 2 * half
+// columns of every q and k head (column i paired with i + half), q to its own
+// tensor, k and v into the paged caches.  y_t = sum_j cw[c][j] u_(t - taps + 1 + j);
+// u at positions before the step's first row of the sequence comes from the
+// sequence's tail state [taps - 1, C], and is zero before position 0.
+struct ConvArgs {
+  void* q_out;  // [T, n_q * d]
+  const void* x;
+  int64_t xs;
+  const float* cw;  // [C, taps]
+  int taps;
+  const void* tail;  // [slots, taps - 1, C]
+  int n_slots;
+  const int64_t* pos;
+  const int64_t* kv_slots;
+  const int* row_seq;   // null (with seq_rows null): row i is sequence i
+  const int* seq_rows;
+  const int* slots;
+  int n_seq, T, n_q, n_k, d, dv;
+  const float* inv_freq;  // [half]
+  int half;
+  void* kc;
+  void* vc;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) conv_rope_cache_kernel(ConvArgs g) {
+  const int t = blockIdx.x;
+  const int C = g.n_q * g.d + g.n_k * (g.d + g.dv);
+  const int s = g.row_seq ? g.row_seq[t] : t;
+  const bool seq_ok = s >= 0 && s < g.n_seq;
+  const int r0 = !seq_ok ? t : (g.seq_rows ? g.seq_rows[s] : t);
+  const int slot = seq_ok ? g.slots[s] : -1;
+  const bool live = slot >= 0 && slot < g.n_slots && r0 >= 0 && r0 <= t;
+  const int64_t p = g.pos[t];
+  const int64_t p0 = p - (t - r0);  // position of the step's first row of this sequence
+  const int m = g.taps - 1;
+  const T* x = (const T*)g.x;
+  const T* tail = (const T*)g.tail + (int64_t)(live ? slot : 0) * m * C;
+  auto conv = [&](int c) -> float {
+    float y = 0.f;
+    for (int jj = 0; jj < g.taps; ++jj) {
+      const int64_t qp = p - m + jj;
+      float u = 0.f;
+      if (qp >= p0) u = ldf<T>(x, (int64_t)(r0 + (qp - p0)) * g.xs + c);
+      else if (qp >= 0) u = ldf<T>(tail, (qp - p0 + m) * C + c);
+      y += g.cw[(int64_t)c * g.taps + jj] * u;
+    }
+    return y;
+  };
+  const int qk = (g.n_q + g.n_k) * g.d;
+  const int64_t kvs = g.kv_slots[t];
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float y = live ? conv(c) : 0.f;
+    if (c < qk) {
+      const int e = c % g.d;
+      if (live && e < 2 * g.half) {
+        const int i = e < g.half ? e : e - g.half;
+        const float other = conv(e < g.half ? c + g.half : c - g.half);
+        float sn, cs;
+        sincosf((float)p * g.inv_freq[i], &sn, &cs);
+        y = e < g.half ? y * cs - other * sn : y * cs + other * sn;
+      }
+      if (c < g.n_q * g.d) stf<T>((T*)g.q_out, (int64_t)t * g.n_q * g.d + c, y);
+      else if (kvs >= 0 && live) stf<T>((T*)g.kc, kvs * (g.n_k * g.d) + (c - g.n_q * g.d), y);
+    } else if (kvs >= 0 && live) {
+      stf<T>((T*)g.vc, kvs * (g.n_k * g.dv) + (c - qk), y);
+    }
+  }
+}
+
+// tail [slots, m, C] <- the last m projected rows of every sequence of the step
+template <typename T>
+__global__ void __launch_bounds__(256) conv_state_update_kernel(T* __restrict__ tail, int n_slots,
+                                                                const T* __restrict__ x, int64_t xs,
+                                                                const int64_t* __restrict__ pos,
+                                                                const int* __restrict__ seq_rows,
+                                                                const int* __restrict__ slots, int T_, int C, int m) {
+  const int s = blockIdx.x;
+  const int r0 = seq_rows ? seq_rows[s] : s, r1 = seq_rows ? seq_rows[s + 1] : s + 1;
+  const int slot = slots[s];
+  const int n = r1 - r0;
+  if (slot < 0 || slot >= n_slots || n <= 0 || r0 < 0 || r1 > T_) return;
+  const int64_t p0 = pos[r0];
+  T* ts = tail + (int64_t)slot * m * C;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    // new[i] is the step-relative row n - m + i: a row of x, or an old entry shifted down.
+    // Ascending i reads old entries at i + n > i only, so a thread may overwrite as it goes.
+    for (int i = 0; i < m; ++i) {
+      const int rel = n - m + i;
+      T val;
+      if (rel >= 0) val = x[(int64_t)(r0 + rel) * xs + c];
+      else if (p0 + rel >= 0) val = ts[(int64_t)(i + n) * C + c];
+      else val = (T)0;
+      ts[(int64_t)i * C + c] = val;
+    }
+  }
+}
+
+// out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate): one wave per (row, head)
+template <typename T>
+__global__ void __launch_bounds__(64) head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                                            const float* __restrict__ w, const T* __restrict__ gate,
+                                                            int64_t gs, int H, int dv, float eps) {
+  const int64_t v = blockIdx.x;
+  const int64_t row = v / H;
+  const int h = (int)(v - row * H);
+  const float* op = o + v * dv;
+  float ss = 0.f;
+  for (int e = threadIdx.x; e < dv; e += 64) ss += op[e] * op[e];
+  const float inv = rsqrtf(wave_reduce_sum(ss) / (float)dv + eps);
+  for (int e = threadIdx.x; e < dv; e += 64) {
+    float y = op[e] * inv;
+    if (w) y *= w[h * dv + e];
+    if (gate) y *= sigmoidf_(ldf<T>(gate, row * gs + h * dv + e));
+    stf<T>(out, v * dv + e, y);
+  }
+}
+
+}  // namespace
+
+#define DISPATCH_T(f32, ...)          \
+  if (f32) {                          \
+    using T = float;                  \
+    __VA_ARGS__;                      \
+  } else {                            \
+    using T = bf16_t;                 \
+    __VA_ARGS__;                      \
+  }
+
+extern "C" {
+
+int dxm_delta_rule(float* out, float* state, int n_slots, const void* r, int64_t rs, const void* k, int64_t ks,
+                   const void* v, int64_t vs, const void* a, int64_t as, const void* w, int64_t ws,
+                   const float* a_bias, const float* w_bias, float decay_scale, float key_eps, const int64_t* pos,
+                   const int* seq_rows, const int* slots, int n_seq, int T_, int H, int dk, int dv, int f32,
+                   hipStream_t st) {
+  if (n_seq <= 0 || T_ <= 0) return 0;
+  if (H < 1 || dk < 1 || dv < 1 || n_slots < 1 || H > 65535 || n_seq > 0x7fffffff) return 1;
+  if (dk > kRows * 16) return 2;  // wider keys need more lanes per column than instantiated
+  if (!out || !state || !pos || !slots) return 3;
+  if (!seq_rows && n_seq != T_) return 4;
+  DeltaArgs g{out, state, r, k, v, a, w, rs, ks, vs, as, ws, a_bias, w_bias, decay_scale, key_eps,
+              pos, seq_rows, slots, n_slots, T_, H, dk, dv};
+  const int need = (dk + kRows - 1) / kRows;
+  if (need <= 1) { DISPATCH_T(f32, (launch_delta<T, 1>(g, n_seq, st))); }
+  else if (need <= 2) { DISPATCH_T(f32, (launch_delta<T, 2>(g, n_seq, st))); }
+  else if (need <= 4) { DISPATCH_T(f32, (launch_delta<T, 4>(g, n_seq, st))); }
+  else if (need <= 8) { DISPATCH_T(f32, (launch_delta<T, 8>(g, n_seq, st))); }
+  else { DISPATCH_T(f32, (launch_delta<T, 16>(g, n_seq, st))); }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw, int taps, const void* tail,
+                        int n_slots, const int64_t* pos, const int64_t* kv_slots, const int* row_seq,
+                        const int* seq_rows, const int* slots, int n_seq, int T_, int n_q, int n_k, int d, int dv,
+                        const float* inv_freq, int half, void* kc, void* vc, int f32, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (taps < 1 || n_q < 0 || n_k < 0 || d < 1 || dv < 0 || half < 0 || 2 * half > d) return 1;
+  if ((half && !inv_freq) || (n_k && (!kc || !vc)) || (taps > 1 && !tail) || !cw || !pos || !kv_slots || !slots)
+    return 2;
+  if ((row_seq == nullptr) != (seq_rows == nullptr) || (!row_seq && n_seq != T_)) return 3;
+  ConvArgs g{q_out, x, xs, cw, taps, tail, n_slots, pos, kv_slots, row_seq, seq_rows, slots, n_seq, T_,
+             n_q, n_k, d, dv, inv_freq, half, kc, vc};
+  DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), 0, st, g));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_conv_state_update(void* tail, int n_slots, const void* x, int64_t xs, const int64_t* pos, const int* seq_rows,
+                          const int* slots, int n_seq, int T_, int C, int taps, int f32, hipStream_t st) {
+  if (n_seq <= 0 || taps <= 1 || C <= 0) return 0;
+  if (!tail || !x || !pos || !slots || (!seq_rows && n_seq != T_)) return 1;
+  const int gy = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
+  DISPATCH_T(f32, hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(n_seq, gy), dim3(256), 0, st, (T*)tail, n_slots,
+                                     (const T*)x, xs, pos, seq_rows, slots, T_, C, taps - 1));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_head_norm_gate(void* out, const float* o, const float* w, const void* gate, int64_t gs, int rows, int H,
+                       int dv, float eps, int f32, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (H < 1 || dv < 1 || (int64_t)rows * H > 0x7fffffff) return 1;
+  DISPATCH_T(f32, hipLaunchKernelGGL(head_norm_gate_kernel<T>, dim3((unsigned)(rows * H)), dim3(64), 0, st, (T*)out, o,
+                                     w, (const T*)gate, gs, H, dv, eps));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // extern "C"

@@ -73,6 +73,10 @@ struct RowAttnArgs {
   float softcap;    // 0: scores are not capped
   const float* r1;  // [n_qh] distance penalty (null: none)
   const float* r2;
+  int wfn;              // 0: softmax over the visible keys; 1: sigmoid(s) per visible key, not normalised
+  const float* hbias;   // [n_qh] added to the score (null: none)
+  const void* gate;     // [rows, gate_stride] logits per head: the result is multiplied by sigmoid (null: none)
+  int64_t gate_stride;
 };
 
 template <typename T, typename OutT, int NV>
@@ -100,7 +104,8 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
   const bool vec = a.d % Elem<T>::kVec == 0 && a.Wk % Elem<T>::kVec == 0;
   const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
   const float r1 = a.r1 ? a.r1[qh] : 0.f, r2 = a.r1 ? a.r2[qh] : 0.f;
-  float mx = -INFINITY, l = 0.f;
+  const float hb = a.hbias ? a.hbias[qh] : 0.f;
+  float mx = a.wfn ? 0.f : -INFINITY, l = a.wfn ? 1.f : 0.f;
   float acc[NV];
 #pragma unroll
   for (int c = 0; c < NV; ++c) acc[c] = 0.f;
@@ -120,15 +125,20 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
       }
       if (cap > 0.f) sum = cap * tanhf(sum * inv_cap);
       if (a.r1) sum -= r1 * log1pf(r2 * (float)(p - j));
-      s = sum;
+      s = sum + hb;
     }
-    const float mn = fmaxf(mx, wave_reduce_max(s));
-    const float w = ok ? __expf(s - mn) : 0.f;
-    const float alpha = __expf(mx - mn);  // first tile: exp(-inf) = 0
-    l = l * alpha + wave_reduce_sum(w);
-    mx = mn;
+    float w;
+    if (a.wfn) {  // every visible key weighs sigmoid(s); nothing to rescale
+      w = ok ? 1.f / (1.f + expf(-s)) : 0.f;
+    } else {
+      const float mn = fmaxf(mx, wave_reduce_max(s));
+      w = ok ? __expf(s - mn) : 0.f;
+      const float alpha = __expf(mx - mn);  // first tile: exp(-inf) = 0
+      l = l * alpha + wave_reduce_sum(w);
+      mx = mn;
 #pragma unroll
-    for (int c = 0; c < NV; ++c) acc[c] *= alpha;
+      for (int c = 0; c < NV; ++c) acc[c] *= alpha;
+    }
     const int64_t left = p - (lo + t * 64) + 1;
     const int n = left < 64 ? (int)left : 64;
     for (int jj = 0; jj < n; ++jj) {
@@ -144,7 +154,8 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
   }
   if (a.parts == 1) {
     OutT* o = (OutT*)a.out + ((int64_t)row * a.n_qh + qh) * a.dv;
-    const float inv = 1.f / l;
+    float inv = 1.f / l;
+    if (a.gate) inv /= 1.f + expf(-Elem<T>::ld((const T*)a.gate, (int64_t)row * a.gate_stride + head));
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
       const int e = lane + 64 * c;
@@ -165,12 +176,22 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
 }
 
 // joins the per-part (max, sum, acc) of one (row, head): one wave each
-template <typename OutT>
+// (sigmoid weights: every part carries max 0 and sum 1, so the join is the plain sum of the
+// parts divided by their number -- `plain` undoes that division); gate: logits [rows, gs] per
+// head, the result is multiplied by their sigmoid
+template <typename OutT, typename GT>
 __global__ void __launch_bounds__(64) merge_parts_kernel(OutT* __restrict__ out, const float* __restrict__ ws,
-                                                         int parts, int dv) {
+                                                         int parts, int dv, int plain, const GT* __restrict__ gate,
+                                                         int64_t gs, int n_qh, int maps) {
   const int lane = threadIdx.x;
   const int64_t v = blockIdx.x;
   const float* w = ws + v * parts * (int64_t)(2 + dv);
+  float post = plain ? (float)parts : 1.f;
+  if (gate) {
+    const int64_t row = v / n_qh;
+    const int head = (int)(v - row * n_qh) / maps;
+    post /= 1.f + expf(-Elem<GT>::ld(gate, row * gs + head));
+  }
   float mx = -INFINITY;
   for (int p = 0; p < parts; ++p) mx = fmaxf(mx, w[(int64_t)p * (2 + dv)]);
   float l = 0.f;
@@ -178,7 +199,7 @@ __global__ void __launch_bounds__(64) merge_parts_kernel(OutT* __restrict__ out,
     const float* wp = w + (int64_t)p * (2 + dv);
     if (wp[1] > 0.f) l += wp[1] * __expf(wp[0] - mx);
   }
-  const float inv = 1.f / l;
+  const float inv = post / l;
   for (int e = lane; e < dv; e += 64) {
     float acc = 0.f;
     for (int p = 0; p < parts; ++p) {
@@ -202,6 +223,7 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
     b.pos = a.pos + r0;
     b.seq = a.seq ? a.seq + r0 : nullptr;
     if (!a.seq && r0) return 5;  // implicit row == sequence numbering cannot be offset
+    b.gate = a.gate ? (const T*)a.gate + (int64_t)r0 * a.gate_stride : nullptr;
     const dim3 grid(a.n_qh, nr, a.parts);
     if (nv <= 1) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 1>), grid, dim3(64), lds, st, b);
     else if (nv <= 2) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 2>), grid, dim3(64), lds, st, b);
@@ -209,8 +231,8 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
     else if (nv <= 8) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 8>), grid, dim3(64), lds, st, b);
     else hipLaunchKernelGGL((row_attention_kernel<T, OutT, 16>), grid, dim3(64), lds, st, b);
     if (a.parts > 1)
-      hipLaunchKernelGGL((merge_parts_kernel<OutT>), dim3((unsigned)nr * a.n_qh), dim3(64), 0, st, (OutT*)b.out, b.ws,
-                         a.parts, a.dv);
+      hipLaunchKernelGGL((merge_parts_kernel<OutT, T>), dim3((unsigned)nr * a.n_qh), dim3(64), 0, st, (OutT*)b.out, b.ws,
+                         a.parts, a.dv, a.wfn, (const T*)b.gate, a.gate_stride, a.n_qh, a.maps);
   }
   DX_CHECK_LAUNCH();
   return 0;
@@ -221,28 +243,35 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
 extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc,
                                  const int64_t* pos, const int* seq, const int* bt, int bt_stride, int bs, int rows,
                                  int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                                 int size, float softcap, const float* r1, const float* r2, int parts, int f32,
-                                 int out_f32, hipStream_t st) {
+                                 int size, float softcap, const float* r1, const float* r2, int wfn, const float* hbias,
+                                 const void* gate, int64_t gate_stride, int parts, int f32, int out_f32,
+                                 hipStream_t st) {
   if (rows <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group) return 1;
   if (d < 1 || dv < 1 || dv > 1024 || d > 8192) return 2;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535 || n_qh > 65535) return 3;
   if (parts > 1 && !ws) return 4;
-  if (softcap < 0.f || (r1 && !r2)) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
   RowAttnArgs a{q, q_stride, kc, vc, out, ws, pos, seq, bt, bt_stride, bs, n_qh, maps, group,
-                d, dv, Wk, Wv, scale, mask, size, parts, softcap, r1, r2};
+                d, dv, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias, gate, gate_stride};
   if (f32) return launch_rows<float, float>(a, rows, st);
   if (out_f32) return launch_rows<bf16_t, float>(a, rows, st);
   return launch_rows<bf16_t, bf16_t>(a, rows, st);
 }
 
-// out [n_vec, dv] (bf16 or fp32) from per-part partials ws [n_vec, parts, 2 + dv]
-extern "C" int dxm_merge_parts(void* out, const float* ws, int64_t n_vec, int parts, int dv, int out_f32,
+// out [n_vec, dv] (bf16 or fp32) from per-part partials ws [n_vec, parts, 2 + dv]; n_vec = rows * n_qh;
+// plain: the parts hold sigmoid-weighted sums (max 0, sum 1 each); gate: bf16 logits [rows, gate_stride]
+extern "C" int dxm_merge_parts(void* out, const float* ws, int64_t n_vec, int parts, int dv, int plain,
+                               const void* gate, int64_t gate_stride, int n_qh, int maps, int out_f32,
                                hipStream_t st) {
   if (n_vec <= 0) return 0;
-  if (parts < 1 || dv < 1 || n_vec > 0x7fffffff) return 1;
-  if (out_f32) hipLaunchKernelGGL((merge_parts_kernel<float>), dim3((unsigned)n_vec), dim3(64), 0, st, (float*)out, ws, parts, dv);
-  else hipLaunchKernelGGL((merge_parts_kernel<bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (bf16_t*)out, ws, parts, dv);
+  if (parts < 1 || dv < 1 || n_vec > 0x7fffffff || n_qh < 1 || maps < 1) return 1;
+  if (out_f32)
+    hipLaunchKernelGGL((merge_parts_kernel<float, bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (float*)out, ws,
+                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps);
+  else
+    hipLaunchKernelGGL((merge_parts_kernel<bf16_t, bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (bf16_t*)out, ws,
+                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps);
   DX_CHECK_LAUNCH();
   return 0;
 }

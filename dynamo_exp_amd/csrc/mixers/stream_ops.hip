@@ -186,17 +186,29 @@ constexpr int kResChunks = 8;
 template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) residual_step_kernel(
     float* __restrict__ X, const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
-    const T* __restrict__ c, int64_t c_stride, const float* __restrict__ cw, float eps, int norm,
-    const float* __restrict__ nw, const float* __restrict__ nb, T* __restrict__ out, T* __restrict__ xc, int W) {
+    const T* __restrict__ c, int64_t c_stride, const float* __restrict__ cw, const T* __restrict__ cg,
+    int64_t cg_stride, const float* __restrict__ cgb, float eps, int norm, const float* __restrict__ nw,
+    const float* __restrict__ nb, T* __restrict__ out, T* __restrict__ xc, int W) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
   float* x = X + row * (int64_t)W;
   float rc = 0.f;
+  // the addend c at columns e .. e + V - 1, gated by sigmoid(cg + cgb) when a gate is given
+  auto load_c = [&](int e, float* v) {
+    ldv<T, V>(c + row * c_stride + e, v);
+    if (cg) {
+      float gt[V], gb[V];
+      ldv<T, V>(cg + row * cg_stride + e, gt);
+      if (cgb) ldv<float, V>(cgb + e, gb);
+#pragma unroll
+      for (int i = 0; i < V; ++i) v[i] *= 1.f / (1.f + expf(-(gt[i] + (cgb ? gb[i] : 0.f))));
+    }
+  };
   if (c) {
     float ss = 0.f;
     for (int e = threadIdx.x * V; e < W; e += kThreads * V) {
       float v[V];
-      ldv<T, V>(c + row * c_stride + e, v);
+      load_c(e, v);
 #pragma unroll
       for (int i = 0; i < V; ++i) ss += v[i] * v[i];
     }
@@ -225,7 +237,7 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
       }
       if (c) {
         float w[V];
-        ldv<T, V>(c + row * c_stride + e, t);
+        load_c(e, t);
         ldv<float, V>(cw + e, w);
 #pragma unroll
         for (int i = 0; i < V; ++i) r[k][i] += t[i] * rc * w[i];
@@ -252,7 +264,7 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
       }
       if (c) {
         float w[V];
-        ldv<T, V>(c + row * c_stride + e, t);
+        load_c(e, t);
         ldv<float, V>(cw + e, w);
 #pragma unroll
         for (int i = 0; i < V; ++i) v[i] += t[i] * rc * w[i];
@@ -313,6 +325,7 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
 }
 
 __device__ __forceinline__ float act_fn(float z, int act) {
+  if (act == 5) return tanhf(z);
   if (act == 0) return fmaxf(z, 0.f);           // relu
   if (act == 1) return z / (1.f + __expf(-z));  // silu
   if (act == 3) return 1.f / (1.f + __expf(-z));  // sigmoid
@@ -330,14 +343,22 @@ __device__ __forceinline__ float act_fn(float z, int act) {
 template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) act_mul_kernel(T* __restrict__ out, const T* __restrict__ gate,
                                                            int64_t g_stride, const T* __restrict__ up,
-                                                           int64_t u_stride, int F, int64_t out_stride, int act) {
+                                                           int64_t u_stride, int F, int64_t out_stride, int act,
+                                                           float limit, float alpha) {
   const int64_t r = blockIdx.y;
   for (int c = (blockIdx.x * kThreads + threadIdx.x) * V; c < F; c += gridDim.x * kThreads * V) {
     float g[V], u[V], o[V];
     ldv<T, V>(gate + r * g_stride + c, g);
     if (up) ldv<T, V>(up + r * u_stride + c, u);
 #pragma unroll
-    for (int e = 0; e < V; ++e) o[e] = act_fn(g[e], act) * (up ? u[e] : 1.f);
+    for (int e = 0; e < V; ++e) {
+      if (act == 6) {  // clamped gated unit: g sigmoid(alpha g) (u + 1), g <= limit, |u| <= limit
+        const float gc = fminf(g[e], limit), uc = fminf(fmaxf(u[e], -limit), limit);
+        o[e] = gc / (1.f + __expf(-alpha * gc)) * (uc + 1.f);
+      } else {
+        o[e] = act_fn(g[e], act) * (up ? u[e] : 1.f);
+      }
+    }
     stv<T, V>(out + r * out_stride + c, o);
   }
 }
@@ -497,23 +518,27 @@ int dxm_gather_rows(void* out, const void* table, const int64_t* ids, int rows, 
 }
 
 int dxm_residual_step(float* X, const void* a, int64_t a_stride, const void* b, int64_t b_stride, const void* c,
-                      int64_t c_stride, const float* cw, float eps, int norm, const float* nw, const float* nb,
-                      void* out, void* xc, int rows, int W, int f32, hipStream_t st) {
+                      int64_t c_stride, const float* cw, const void* cg, int64_t cg_stride, const float* cgb, float eps,
+                      int norm, const float* nw, const float* nb, void* out, void* xc, int rows, int W, int f32,
+                      hipStream_t st) {
   if (rows <= 0) return 0;
   if (W < 1 || norm < 0 || norm > 2) return 1;
-  if ((c && !cw) || (norm && (!nw || !out)) || (norm == 2 && !nb)) return 2;
+  if ((c && !cw) || (norm && (!nw || !out)) || (norm == 2 && !nb) || (cg && !c)) return 2;
   const int esz = f32 ? 4 : 2;
   auto al = [&](const void* p, int by) { return (uintptr_t)p % by == 0; };
-  const bool vec = W % 4 == 0 && a_stride % 4 == 0 && b_stride % 4 == 0 && c_stride % 4 == 0 && al(X, 16) &&
-                   al(a, 4 * esz) && al(b, 4 * esz) && al(c, 4 * esz) && al(cw, 16) && al(nw, 16) && al(nb, 16) &&
+  const bool vec = W % 4 == 0 && a_stride % 4 == 0 && b_stride % 4 == 0 && c_stride % 4 == 0 && cg_stride % 4 == 0 &&
+                   al(X, 16) && al(a, 4 * esz) && al(b, 4 * esz) && al(c, 4 * esz) && al(cg, 4 * esz) && al(cgb, 16) &&
+                   al(cw, 16) && al(nw, 16) && al(nb, 16) &&
                    al(out, 4 * esz) && al(xc, 4 * esz);
   if (vec) {
     DISPATCH_T(f32, hipLaunchKernelGGL((residual_step_kernel<T, 4>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)a,
-                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, eps, norm, nw, nb,
+                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, (const T*)cg, cg_stride, cgb, eps,
+                                       norm, nw, nb,
                                        (T*)out, (T*)xc, W));
   } else {
     DISPATCH_T(f32, hipLaunchKernelGGL((residual_step_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)a,
-                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, eps, norm, nw, nb,
+                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, (const T*)cg, cg_stride, cgb, eps,
+                                       norm, nw, nb,
                                        (T*)out, (T*)xc, W));
   }
   DX_CHECK_LAUNCH();
@@ -521,9 +546,9 @@ int dxm_residual_step(float* X, const void* a, int64_t a_stride, const void* b, 
 }
 
 int dxm_act_mul(void* out, const void* gate, int64_t g_stride, const void* up, int64_t u_stride, int rows, int F,
-                int64_t out_stride, int act, int f32, hipStream_t st) {
+                int64_t out_stride, int act, float limit, float alpha, int f32, hipStream_t st) {
   if (rows <= 0 || F <= 0) return 0;
-  if (act < 0 || act > 4) return 1;
+  if (act < 0 || act > 6 || (act == 6 && (!up || !(limit > 0.f)))) return 1;
   const int esz = f32 ? 4 : 2;
   const bool vec = F % 4 == 0 && g_stride % 4 == 0 && u_stride % 4 == 0 && out_stride % 4 == 0 &&
                    (uintptr_t)gate % (4 * esz) == 0 && (uintptr_t)up % (4 * esz) == 0 &&
@@ -535,11 +560,13 @@ int dxm_act_mul(void* out, const void* gate, int64_t g_stride, const void* up, i
     if (vec) {
       DISPATCH_T(f32, hipLaunchKernelGGL((act_mul_kernel<T, 4>), dim3(gx, nr), dim3(kThreads), 0, st,
                                          (T*)out + r0 * out_stride, (const T*)gate + r0 * g_stride, g_stride,
-                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act));
+                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act,
+                                         limit, alpha));
     } else {
       DISPATCH_T(f32, hipLaunchKernelGGL((act_mul_kernel<T, 1>), dim3(gx, nr), dim3(kThreads), 0, st,
                                          (T*)out + r0 * out_stride, (const T*)gate + r0 * g_stride, g_stride,
-                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act));
+                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act,
+                                         limit, alpha));
     }
   }
   DX_CHECK_LAUNCH();

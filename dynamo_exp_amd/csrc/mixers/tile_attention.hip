@@ -50,6 +50,10 @@ struct TileArgs {
   float softcap;    // 0: none
   const float* r1;  // [n_qh], null: no distance penalty
   const float* r2;
+  int wfn;             // 0: softmax; 1: sigmoid(s + hbias) per visible key, not normalised
+  const float* hbias;  // [n_qh] (sigmoid weights only; a constant per head leaves a softmax unchanged)
+  const bf16_t* gate;  // [rows, gate_stride] logits per head: the result is multiplied by their sigmoid
+  int64_t gate_stride;
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -219,6 +223,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
   const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
   const float r1 = a.r1 ? a.r1[qh] : 0.f, r2 = a.r1 ? a.r2[qh] : 0.f;
   const float sc2 = terms ? 1.f : a.scale * kLog2e;  // scores in log2 units: exp2 is one instruction
+  const float hb2 = a.hbias ? a.hbias[qh] * kLog2e : 0.f;
   float mx[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
   f32x4 O[2][DVB];
 #pragma unroll
@@ -274,6 +279,31 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
       const bool full = 32 * w + 31 < n && kt + kKeys - 1 <= p0 + 32 * w &&
                         kt >= first_visible(p0 + 32 * w + 31, a.mask, a.size);
       i16x4 Ph[2][4], Pl[2][4];
+      if (a.wfn) {
+        // sigmoid weights: w = 1 / (1 + 2^-(x log2 e)), x = s + hbias; invisible keys weigh 0;
+        // no maximum, no rescaling, no normalisation
+        const float xs = terms ? 1.f : a.scale * kLog2e;
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb) {
+            float p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int kj = kt + kb * 16 + 4 * g4 + i;
+              const bool vis = full || (okrow[qb] && kj >= lrow[qb] && kj <= prow[qb]);
+              const float w_ = __builtin_amdgcn_rcpf(1.f + fast_exp2(-fmaf(S[qb][kb][i], xs, hb2)));
+              p[i] = vis ? w_ : 0.f;
+            }
+            const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
+            Ph[qb][kb] = __builtin_bit_cast(i16x4, uint2{h01, h23});
+            if constexpr (kHiLo) {
+              const uint32_t l01 = pack_bf16x2(p[0] - bf16lo(h01), p[1] - bf16hi(h01));
+              const uint32_t l23 = pack_bf16x2(p[2] - bf16lo(h23), p[3] - bf16hi(h23));
+              Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
+            }
+          }
+      } else {
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb) {
         // scale > 0 (checked on the host): the row maximum is taken over the raw sums and
@@ -328,6 +358,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
           lsum[qb] += add;
         }
       }
+      }
 #pragma unroll
       for (int kp = 0; kp < 2; ++kp) {  // 32 keys per MFMA: key blocks 2 kp and 2 kp + 1
         bf16x8_t Bh[2], Bl[2];
@@ -356,8 +387,9 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!okrow[qb]) continue;
-    const float inv = 1.f / l;
     const int r = 32 * w + 16 * qb + c16;
+    float inv = a.wfn ? 1.f : 1.f / l;
+    if (a.gate) inv /= 1.f + __expf(-bf16_to_f32(a.gate[(int64_t)(row0 + r) * a.gate_stride + head]));
     OutT* o = (OutT*)a.out + ((int64_t)(row0 + r) * a.n_qh + qh) * dv + 4 * g4;
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb) store4<OutT>(o + cb * 16, O[qb][cb] * inv);
@@ -389,6 +421,8 @@ struct GroupArgs {
   float softcap;
   const float* r1;
   const float* r2;
+  int wfn;
+  const float* hbias;
 };
 
 template <int DB, int DVB, int QB>
@@ -413,7 +447,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   i16x4 qf[QB][DB];
   bool okh[QB];
   int qh[QB];
-  float r1[QB], r2[QB];
+  float r1[QB], r2[QB], hb[QB];
   const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
@@ -422,6 +456,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
     qh[qb] = (g * a.group + (okh[qb] ? hi_ : 0)) * a.maps + m;
     r1[qb] = a.r1 ? a.r1[qh[qb]] : 0.f;
     r2[qb] = a.r1 ? a.r2[qh[qb]] : 0.f;
+    hb[qb] = a.hbias ? a.hbias[qh[qb]] : 0.f;
     const bf16_t* q = a.q + (int64_t)row * a.q_stride + (int64_t)qh[qb] * d + 4 * g4;
 #pragma unroll
     for (int ks = 0; ks < DB; ++ks)
@@ -431,7 +466,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   f32x4 O[QB][DVB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    mx[qb] = -INFINITY;
+    mx[qb] = a.wfn ? 0.f : -INFINITY;  // sigmoid weights: every part reports max 0 and sum 1
     lsum[qb] = 0.f;
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -478,14 +513,14 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
           float s = S[qb][kb][i] * a.scale;
           if (cap > 0.f) s = cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * s * inv_cap)));
           if (a.r1) s -= r1[qb] * __logf(1.f + r2[qb] * (float)(p - kj > 0 ? p - kj : 0));
-          s = kj <= p ? s : -INFINITY;
+          s = kj <= p ? s + hb[qb] : -INFINITY;
           S[qb][kb][i] = s;
           mloc = fmaxf(mloc, s);
         }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-      const float mn = fmaxf(mx[qb], mloc);  // finite: every visited tile holds a visible key
-      const float alpha = __expf(mx[qb] - mn);
+      const float mn = a.wfn ? 0.f : fmaxf(mx[qb], mloc);  // finite: every visited tile holds a visible key
+      const float alpha = __expf(mx[qb] - mn);              // sigmoid weights: 1
       mx[qb] = mn;
       float add = 0.f;
 #pragma unroll
@@ -493,7 +528,8 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
         float pw[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          pw[i] = __expf(S[qb][kb][i] - mn);
+          // sigmoid(s); an invisible key (s = -inf) weighs 1 / (1 + inf) = 0
+          pw[i] = a.wfn ? __builtin_amdgcn_rcpf(1.f + __expf(-S[qb][kb][i])) : __expf(S[qb][kb][i] - mn);
           add += pw[i];
         }
         const uint32_t h01 = pack_bf16x2(pw[0], pw[1]), h23 = pack_bf16x2(pw[2], pw[3]);
@@ -528,7 +564,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
     float* w = a.ws + (((int64_t)row * a.n_qh + qh[qb]) * a.parts + part) * (2 + dv);
     if (g4 == 0) {
       w[0] = mx[qb];
-      w[1] = l;
+      w[1] = a.wfn ? 1.f : l;
     }
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb)
@@ -603,14 +639,16 @@ int dxm_tile_attention_ok(int d, int dv) {
 int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
                        const int* seq, const int* bt, int bt_stride, int bs, const int* tiles, int n_tiles, int n_qh,
                        int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask, int size,
-                       float softcap, const float* r1, const float* r2, int out_f32, hipStream_t st) {
+                       float softcap, const float* r1, const float* r2, int wfn, const float* hbias, const void* gate,
+                       int64_t gate_stride, int out_f32, hipStream_t st) {
   if (n_tiles <= 0) return 0;
-  if (softcap < 0.f || (r1 && !r2)) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || !(scale > 0.f)) return 3;
   if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 8) return 4;
   TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
-             tiles, n_qh, maps, group, Wk, Wv, scale, mask, size, softcap, r1, r2};
+             tiles, n_qh, maps, group, Wk, Wv, scale, mask, size, softcap, r1, r2, wfn, hbias, (const bf16_t*)gate,
+             gate_stride};
   TILE_CASE(2, 2)
   TILE_CASE(3, 3)
   TILE_CASE(3, 6)
@@ -630,14 +668,14 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
 int dxm_group_decode(float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
                      const int* seq, const int* bt, int bt_stride, int bs, int rows, int n_qh, int maps, int group,
                      int d, int dv, int Wk, int Wv, float scale, int mask, int size, float softcap, const float* r1,
-                     const float* r2, int parts, hipStream_t st) {
+                     const float* r2, int wfn, const float* hbias, int parts, hipStream_t st) {
   if (rows <= 0) return 0;
-  if (softcap < 0.f || (r1 && !r2)) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || rows > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535) return 3;
   if (!ws || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
   GroupArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, ws, pos, seq, bt, bt_stride, bs,
-              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts, softcap, r1, r2};
+              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias};
   GROUP_CASE(2, 2)
   GROUP_CASE(3, 3)
   GROUP_CASE(3, 6)

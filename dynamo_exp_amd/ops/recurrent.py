@@ -169,7 +169,9 @@ def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tenso
                seq_rows: torch.Tensor | None, state_slots: torch.Tensor, n_heads: int, dk: int, dv: int,
                decay_scale: float = DELTA_DECAY_SCALE, key_eps: float = 1e-6) -> torch.Tensor:
     """The generalized delta rule over the rows of a step, per sequence and head
-    from the sequence's state S [dk, dv] (fp32, state [slots, H, dk, dv],
+    from the sequence's state S [dk, dv] (fp32; stored column by column,
+    state [slots, H, dv, dk] with state[s, h, j, i] = S[i, j], so that the
+    kernel's threads, which own columns, read and write contiguous runs;
     updated in place):
         decay   w_t = exp(-decay_scale * sigmoid(w + w_bias))       per key channel
         removal a_t = sigmoid(a + a_bias)                           per key channel
@@ -187,8 +189,8 @@ def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tenso
     for t, wd in ((r, dk), (k, dk), (a, dk), (w, dk), (v, dv)):
         if t.shape != (T, n_heads * wd) or t.stride(1) != 1 or t.dtype != r.dtype:
             raise ValueError("delta_rule: r, k, a, w [T, H dk] and v [T, H dv] with contiguous rows, one dtype")
-    if state.shape[1:] != (n_heads, dk, dv) or state.dtype != torch.float32 or not state.is_contiguous():
-        raise ValueError("delta_rule: state is contiguous float32 [slots, H, dk, dv]")
+    if state.shape[1:] != (n_heads, dv, dk) or state.dtype != torch.float32 or not state.is_contiguous():
+        raise ValueError("delta_rule: state is contiguous float32 [slots, H, dv, dk]")
     if not r.is_cuda:
         out = torch.zeros((T, n_heads, dv), dtype=torch.float32)
         H = n_heads
@@ -202,13 +204,14 @@ def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tenso
             sl = int(state_slots[s])
             if sl < 0 or r1 <= r0:
                 continue
-            S = state[sl].clone() if int(positions[r0]) > 0 else torch.zeros_like(state[sl])
+            S = state[sl].transpose(1, 2).clone() if int(positions[r0]) > 0 else \
+                torch.zeros((H, dk, dv), dtype=torch.float32)
             for t in range(r0, r1):
                 uS = torch.einsum("hi,hij->hj", uf[t], S)
                 S = wf[t][:, :, None] * S - (af[t] * uf[t])[:, :, None] * uS[:, None, :] + \
                     kf[t][:, :, None] * vf[t][:, None, :]
                 out[t] = torch.einsum("hi,hij->hj", rf[t], S)
-            state[sl] = S
+            state[sl] = S.transpose(1, 2)
         return out.view(T, H * dv)
     out = torch.empty((T, n_heads * dv), dtype=torch.float32, device=r.device)
     _m().delta_rule(out.data_ptr(), state.data_ptr(), state.shape[0], r.data_ptr(), r.stride(0), k.data_ptr(),
