@@ -1,6 +1,7 @@
-"""`bench.py --layered`: the layer-listed models (Bekulix, Bolinex) beside the
-closest existing model (Llama) at equal layer sizes, random weights.
-`--layered-family` picks which of the two families runs (default both).
+"""`bench.py --layered`: the layer-listed models (Bekulix, Bolinex, Nefivik) beside
+the closest existing model (Llama; for Nefivik also Bolinex, the closest
+layer-listed one) at equal layer sizes, random weights.
+`--layered-family` picks which family runs (default: Bekulix and Bolinex).
 
 Two parts, both on one GPU:
   * engine throughput through the engine's own entry point (add_request +
@@ -23,9 +24,10 @@ import torch
 from .. import ops
 from ..engine.engine import EngineConfig, LLMEngine
 from ..engine.request import SamplingParams
-from ..models.config import ModelConfig, _bekulix_preset, _bolinex_preset
+from ..models.config import ModelConfig, _bekulix_preset, _bolinex_preset, _nefivik_preset
 from ..ops import mixers as mx
 from ..ops import moe
+from ..ops import recurrent as rc
 
 # layer sizes of real models (width, ff, heads, kv heads, head dim), a few layers each
 SIZES = {
@@ -49,6 +51,15 @@ def _bolinex_config(s: dict):
     return _bolinex_preset(f"bolinex {s['W']}", s["W"], s["ff"], s["layers"], s["H"], s["G"], s["d"], 1024, experts=8,
                            top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 4, groups=(4, 2), side=256,
                            vocab=s["vocab"])
+
+
+def _nefivik_config(s: dict):
+    """Nefivik at the size's layer shapes: three generalized-delta-rule layers, then a windowed
+    (1024) sigmoid-attention layer with 4-tap convolutions, twice; the second attention layer
+    reads the first one's keys and values; every feed-forward routes 2 of 8 experts of a quarter
+    of the dense width (two of four groups kept); token input of 256 columns."""
+    return _nefivik_preset(f"nefivik {s['W']}", s["W"], s["layers"], s["H"], s["G"], s["d"], 1024, experts=8, top=2,
+                           expert_ff=s["ff"] // 4, groups=(4, 2), side=256, vocab=s["vocab"], conv=4, attn_every=4)
 
 
 def _timed(fn, iters=10, warm=2) -> float:
@@ -300,6 +311,115 @@ def bolinex_kernels(s: dict, L: int, B: int, T: int) -> dict:
     return res
 
 
+def nefivik_kernels(s: dict, L: int, B: int, T: int) -> dict:
+    """Nefivik's kernels alone, each beside its counterpart where there is one: the delta-rule
+    scan over 4 prompts of L / 2 tokens (tokens/s, and the bytes of its inputs and outputs) and
+    over B decode rows (TB/s of the state read and written); convolution + rotation + cache
+    write against Llama's rope_cache; sigmoid-weight window attention against the same kernels
+    with softmax; the gated residual step against Llama's add + RMS norm; the clamped gated
+    unit against silu_and_mul; the softmax router."""
+    H, G, d, W, ff, bs = s["H"], s["G"], s["d"], s["W"], s["ff"], 64
+    dev, dt, win = "cuda", torch.bfloat16, 1024
+    res = {}
+
+    def put(name, us, byts=None, flops=None, **kw):
+        res[name] = {"us": round(us, 1), **kw}
+        if byts:
+            res[name]["TB/s"] = round(byts / us / 1e6, 2)
+        if flops:
+            res[name]["TFLOPs"] = round(flops / us / 1e6, 1)
+
+    # ---- delta rule: prompts, then decode rows
+    n = H * d
+    for tag, n_seq, rows in (("prefill", 4, L // 2), ("decode", B, 1)):
+        Tn = n_seq * rows
+        p = torch.randn(Tn, 5 * n, device=dev, dtype=dt)
+        wl = torch.randn(Tn, n, device=dev, dtype=dt)
+        ab, wb = torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+        state = torch.zeros(n_seq, H, d, d, device=dev)
+        pos = (torch.arange(rows, device=dev) + 1).repeat(n_seq)
+        seq_rows = torch.arange(0, Tn + 1, rows, dtype=torch.int32, device=dev) if rows > 1 else None
+        slots = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        us = _timed(lambda: rc.delta_rule(p[:, :n], p[:, n:2 * n], p[:, 2 * n:3 * n], p[:, 3 * n:4 * n], wl, ab, wb, state,
+                                          pos, seq_rows, slots, H, d, d))
+        io = Tn * n * (5 * 2 + 4)  # five bf16 inputs, fp32 output
+        st = n_seq * H * d * d * 4 * 2  # state read and written
+        put(f"delta_rule_{tag}", us, io + st, 2.0 * 4 * Tn * H * d * d, tok_per_s=round(Tn / us * 1e6),
+            state_TBs=round(st / us / 1e6, 2))
+        o = torch.randn(Tn, n, device=dev)
+        hw = torch.ones(n, device=dev)
+        put(f"head_norm_gate_{tag}", _timed(lambda: rc.head_norm_gate(o, H, hw, p[:, 4 * n:5 * n], 1e-5, dt)),
+            Tn * n * (4 + 2 + 2))
+    # ---- convolution + rotation + cache write
+    taps, C = 4, (H + 2 * G) * d
+    x = torch.randn(T, C, device=dev, dtype=dt)
+    cw = torch.randn(C, taps, device=dev)
+    tail = torch.zeros(1, taps - 1, C, device=dev, dtype=dt)
+    nbt = T // bs + 1
+    kc = torch.zeros(nbt * bs, G * d, device=dev, dtype=dt)
+    vc = torch.zeros_like(kc)
+    posT = torch.arange(T, device=dev)
+    rs = torch.zeros(T, dtype=torch.int32, device=dev)
+    sr = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    s0 = torch.zeros(1, dtype=torch.int32, device=dev)
+    inv = rc.rotary_frequencies(d // 2, 500000.0, None).to(dev)
+    put("conv_rope_cache", _timed(lambda: rc.conv_rope_cache(x, cw, tail, posT, posT, rs, sr, s0, H, G, d, d, inv, kc, vc)),
+        T * d * 2 * (2 * H + 4 * G))
+    qkv = torch.randn(T, C, device=dev, dtype=dt)
+    from ..ops import reference as ref
+    cs = ref.rope_cos_sin(d, T + 1, 500000.0, None).to(dev)
+    kl = torch.zeros(nbt, G, bs, d, device=dev, dtype=dt)
+    vl = torch.zeros_like(kl)
+    put("llama_rope_cache", _timed(lambda: ops.rope_cache(qkv, posT, cs, posT, kl, vl, H, G, d, bs)),
+        T * d * 2 * (2 * H + 4 * G))
+    # ---- window attention: sigmoid weights + head bias + head gate against softmax
+    nb = L // bs + 1
+    q = torch.randn(L, H * d, device=dev, dtype=dt)
+    pos = torch.arange(L, device=dev)
+    seq = torch.zeros(L, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
+    kc = torch.randn(nb * bs, G * d, device=dev, dtype=dt)
+    vc = torch.randn_like(kc)
+    tiles = torch.tensor(mx.tile_list(0, L), dtype=torch.int32, device=dev)
+    pb = torch.randn(H, device=dev) - 3
+    gate = torch.randn(L, H, device=dev, dtype=dt)
+    j = torch.arange(L)
+    fl = 4 * d * H * float((j - mx.first_visible(j, "window", win) + 1).sum())
+    for name, kw in (("softmax", {}), ("sigmoid_gate", dict(weights="sigmoid", head_bias=pb, head_gate=gate))):
+        us = _timed(lambda: mx.attention(q, kc, vc, pos, seq, bt, bs, H, 1, H // G, d, d, d ** -0.5, "window", win, 1,
+                                         False, tiles, L, **kw))
+        put(f"prefill_window{win}_{name}", us, None, fl)
+    nbb = B * nb
+    byts = B * min(L, win) * G * d * 2 * 2
+    btd = torch.randperm(nbb, device=dev).to(torch.int32).view(B, nb)
+    kcd = torch.randn(nbb * bs, G * d, device=dev, dtype=dt)
+    vcd = torch.randn_like(kcd)
+    qd = torch.randn(B, H * d, device=dev, dtype=dt)
+    posd = torch.full((B,), L - 1, device=dev)
+    parts = mx.row_attention_parts(B, G, win, mx.GROUP_TARGET_WAVES)
+    for name, kw in (("softmax", {}), ("sigmoid_gate", dict(weights="sigmoid", head_bias=pb, head_gate=gate[:B]))):
+        us = _timed(lambda: mx.attention(qd, kcd, vcd, posd, None, btd, bs, H, 1, H // G, d, d, d ** -0.5, "window", win,
+                                         parts, **kw))
+        put(f"decode_window{win}_{name}", us, byts, parts=parts)
+    # ---- row kernels
+    X = torch.randn(T, W, device=dev)
+    c, g = torch.randn(T, W, device=dev, dtype=dt), torch.randn(T, W, device=dev, dtype=dt)
+    nw = torch.ones(W, device=dev)
+    put("residual_step_gated_unit_rms_addend_rmsnorm",
+        _timed(lambda: mx.residual_step(X, c=c, c_w=nw, eps=1e-5, norm="rms", norm_w=nw, out_dtype=dt, c_gate=g,
+                                        c_gate_b=nw)), T * W * (4 + 4 + 2 + 2 + 2))
+    a, r = torch.randn(T, W, device=dev, dtype=dt), torch.randn(T, W, device=dev, dtype=dt)
+    w16 = torch.ones(W, device=dev, dtype=dt)
+    put("llama_add_rmsnorm", _timed(lambda: ops.add_rmsnorm(a, r, w16, 1e-6)), T * W * 2 * 4)
+    fe = ff // 4
+    gu = torch.randn(2 * T, 2 * fe, device=dev, dtype=dt)
+    put("glu_act_swiglu_clamp", _timed(lambda: mx.glu_act(gu, "swiglu_clamp", 7.0, 1.702)), 2 * T * fe * 2 * 3)
+    put("llama_silu_and_mul", _timed(lambda: ops.silu_and_mul(gu)), 2 * T * fe * 2 * 3)
+    z = torch.randn(T, 8, device=dev)
+    put("moe_route_softmax", _timed(lambda: moe.route(z, None, 2, 4, 2, score="softmax", group_score="max")))
+    return res
+
+
 def run_layered_compare(args, dev) -> dict:
     isl, osl = min(args.isl, 2048), min(args.osl, 64)
     fam = getattr(args, "layered_family", "all")
@@ -312,11 +432,18 @@ def run_layered_compare(args, dev) -> dict:
         if fam in ("all", "bolinex"):
             row["bolinex"] = engine_throughput(_bolinex_config(s), dev, isl, osl, 4, 64, args.seed)
             row["bolinex_kernels"] = bolinex_kernels(s, 4096, 64, 8192)
+        if fam == "nefivik":
+            row["nefivik"] = engine_throughput(_nefivik_config(s), dev, isl, osl, 4, 64, args.seed)
+            row["nefivik_kernels"] = nefivik_kernels(s, 4096, 64, 8192)
+            row["bolinex"] = engine_throughput(_bolinex_config(s), dev, isl, osl, 4, 64, args.seed)
         row["llama"] = engine_throughput(lla, dev, isl, osl, 4, 64, args.seed)
+        if fam == "nefivik":
+            sizes[name] = row
+            continue
         row["attention_kernels"] = attention_kernels(s, 4096, 64)
         if fam in ("all", "bekulix"):
             row["rowwise_kernels"] = rowwise_kernels(s, 8192)
         sizes[name] = row
-    return {"metric": "layer-listed models (Bekulix, Bolinex) beside Llama at equal layer sizes: engine prefill / "
+    return {"metric": "layer-listed models (Bekulix, Bolinex, Nefivik) beside Llama at equal layer sizes: engine prefill / "
                       "decode tokens/s and kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
             "family": fam, "data": "synthetic (random-token prompts, random-init weights)", "sizes": sizes}

@@ -155,9 +155,11 @@ def attention(h, W, p, m, kv):
 
 
 # ----------------------------------------------------------------- feed-forward
-def route(h, Wr, r):
+def route(h, Wr, r, gaps=None):
     """(chosen experts [T, top], their weights): softmax scores; groups ranked by
-    their best score; the top scores among the kept groups; weights are the scores."""
+    their best score; the top scores among the kept groups; weights are the scores.
+    gaps collects, per token, how far the weakest choice (expert or group) is ahead
+    of the strongest one not chosen."""
     s = torch.softmax(h @ Wr.T, -1)
     T, E = s.shape
     c = s.clone()
@@ -168,7 +170,13 @@ def route(h, Wr, r):
         kept = torch.zeros(T, gr["count"], dtype=torch.bool)
         kept.scatter_(1, gs.topk(gr["keep"], -1).indices, True)
         c = c.masked_fill(~kept.repeat_interleave(per, 1), -1.0)
+        if gaps is not None and gr["keep"] < gr["count"]:
+            g2 = gs.topk(gr["keep"] + 1, -1).values
+            gaps.append(g2[:, -2] - g2[:, -1])
     idx = c.topk(r["top"], -1).indices
+    if gaps is not None and r["top"] < E:
+        c2 = c.topk(r["top"] + 1, -1).values
+        gaps.append(torch.where(c2[:, -1] >= 0, c2[:, -2] - c2[:, -1], torch.ones(T, dtype=F)))
     return idx, s.gather(1, idx)
 
 
@@ -178,8 +186,8 @@ def expert(h, Wg, Wu, Wd, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ Wd.T
 
 
-def moe(h, W, p, mlp):
-    idx, wts = route(h, W[p + "router"], mlp["router"])
+def moe(h, W, p, mlp, gaps=None):
+    idx, wts = route(h, W[p + "router"], mlp["router"], gaps)
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
         for e, w in zip(idx[t].tolist(), wts[t]):
@@ -194,8 +202,9 @@ def token_input(x, e, W, p, eps):
     return unit_rms(y, eps) * W[p + "norm"]
 
 
-def forward(cfg: dict, W: dict, toks: list[int], layers_out: list | None = None):
-    """Logits [T, vocab] of one sequence; layers_out collects the residual after every layer."""
+def forward(cfg: dict, W: dict, toks: list[int], layers_out: list | None = None, gaps: list | None = None):
+    """Logits [T, vocab] of one sequence; layers_out collects the residual after every layer,
+    gaps the margins of every routing decision ([T] each)."""
     W = {k: v.to(F) if v.is_floating_point() else v for k, v in W.items()}
     eps = cfg["norm"]["eps"]
     side = (cfg.get("token_side") or {}).get("dim", 0)
@@ -217,7 +226,7 @@ def forward(cfg: dict, W: dict, toks: list[int], layers_out: list | None = None)
         x = x + rms_norm(y, W[p + "norm1b"], eps)
         if L.get("mlp"):
             h = rms_norm(x, W[p + "norm2"], eps)
-            y = moe(h, W, p + "mlp.", L["mlp"])
+            y = moe(h, W, p + "mlp.", L["mlp"], gaps)
             y = y * sigmoid(h @ W[p + "rg2"].T + W[p + "rg2.b"])
             x = x + rms_norm(y, W[p + "norm2b"], eps)
         if side:
