@@ -353,7 +353,7 @@ def nefivik_kernels(s: dict, L: int, B: int, T: int) -> dict:
     # ---- convolution + rotation + cache write
     taps, C = 4, (H + 2 * G) * d
     x = torch.randn(T, C, device=dev, dtype=dt)
-    cw = torch.randn(C, taps, device=dev)
+    cw = torch.randn(taps, C, device=dev)
     tail = torch.zeros(1, taps - 1, C, device=dev, dtype=dt)
     nbt = T // bs + 1
     kc = torch.zeros(nbt * bs, G * d, device=dev, dtype=dt)

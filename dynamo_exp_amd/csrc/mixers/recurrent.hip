@@ -30,18 +30,19 @@ __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-
 //     S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,   o_t = S_t^T r_t
 // with w_t = exp(-decay_scale * sigmoid(wl_t + w_bias)), a_t = sigmoid(al_t + a_bias),
 // u_t = k_t / sqrt(sum(k_t^2) + key_eps).  Columns of S are independent, so a
-// thread owns kRows consecutive rows of one column in registers, R threads
-// (neighbouring lanes) share a column and join their partial dot products by
-// lane exchanges, and a workgroup of 256 threads owns 256 / R columns of one
-// (sequence, head).  The state tensor is stored column-major per head
-// ([slots, H, dv, dk]) so that a wave's state traffic is one contiguous run.
-// Tokens are staged through LDS kTok at a time: raw r, k, a, w, v rows are
-// fetched into registers one block ahead (their latency hides behind the
-// current block's recurrence), committed, transformed in place (sums of
-// squares by wave reductions), and consumed token by token.
+// thread owns a tile of kRows consecutive rows x kCols consecutive columns in
+// registers (every row vector it reads from LDS serves kCols columns), R
+// neighbouring lanes share the columns and join their partial dot products by
+// DPP lane exchanges (no LDS traffic), and a workgroup of NT threads owns
+// NT / R * kCols columns of one (sequence, head).  The state tensor is stored
+// column-major per head ([slots, H, dv, dk]) so that a wave's state traffic is
+// contiguous runs.  Tokens are staged through LDS kTok at a time: raw r, k, a,
+// w, v rows are fetched into registers one block ahead (their latency hides
+// behind the current block's recurrence), committed, transformed in place
+// (sums of squares by wave reductions), and consumed token by token.
 constexpr int kRows = 16;  // state rows per thread
+constexpr int kCols = 4;   // state columns per thread
 constexpr int kTok = 8;    // tokens per staged block
-constexpr int kDThreads = 256;
 
 struct DeltaArgs {
   float* out;    // [T, H * dv]
@@ -57,61 +58,80 @@ struct DeltaArgs {
   int n_slots, T, H, dk, dv;
 };
 
-template <typename T, int R>
-__global__ void __launch_bounds__(kDThreads) delta_rule_kernel(DeltaArgs g) {
-  constexpr int kCols = kDThreads / R;      // columns per workgroup
-  constexpr int kDkp = kRows * R;           // padded key width
-  constexpr int kE = (kTok * kDkp + kDThreads - 1) / kDThreads;   // staged elements per thread and array
-  constexpr int kEv = (kTok * kCols + kDThreads - 1) / kDThreads;
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+// sum over the R lanes of an aligned lane group (R <= 16), the result in every lane of the group:
+// neighbours within a quad, the other pair of the quad, the other quad of a half row (half-row
+// mirror: the quads already hold one value each), the other half of a row of 16 (row mirror)
+template <int R> __device__ __forceinline__ float group_sum(float v) {
+  if constexpr (R >= 2) v += dpp_f<0xB1>(v);
+  if constexpr (R >= 4) v += dpp_f<0x4E>(v);
+  if constexpr (R >= 8) v += dpp_f<0x141>(v);
+  if constexpr (R >= 16) v += dpp_f<0x140>(v);
+  return v;
+}
+
+template <typename T, int R, int NT>
+__global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
+  constexpr int kGroups = NT / R;            // column tiles per workgroup
+  constexpr int kWgCols = kGroups * kCols;   // columns per workgroup
+  constexpr int kDkp = kRows * R;            // padded key width
+  constexpr int kE = (kTok * kDkp + NT - 1) / NT;  // staged elements per thread and array
+  constexpr int kEv = (kTok * kWgCols + NT - 1) / NT;
   __shared__ __attribute__((aligned(16))) float sr[kTok][kDkp];
   __shared__ __attribute__((aligned(16))) float sk[kTok][kDkp];
   __shared__ __attribute__((aligned(16))) float su[kTok][kDkp];
   __shared__ __attribute__((aligned(16))) float sw[kTok][kDkp];
   __shared__ __attribute__((aligned(16))) float sa[kTok][kDkp];
-  __shared__ float sv[kTok][kCols];
-  const int tid = threadIdx.x, part = tid % R, c = tid / R;
-  const int s = blockIdx.x, h = blockIdx.y, j = blockIdx.z * kCols + c;
+  __shared__ __attribute__((aligned(16))) float sv[kTok][kWgCols];
+  const int tid = threadIdx.x, part = tid % R, grp = tid / R;
+  const int s = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * kWgCols + grp * kCols;
   const int r0 = g.seq_rows ? g.seq_rows[s] : s;
   const int r1 = g.seq_rows ? g.seq_rows[s + 1] : s + 1;
   const int slot = g.slots[s];
   const int n = r1 - r0;
   if (n <= 0 || r0 < 0 || r1 > g.T) return;
-  const bool col_ok = j < g.dv;
   if (slot < 0 || slot >= g.n_slots) {  // padding rows: a defined result, no state
-    if (col_ok && part == 0)
-      for (int t = r0; t < r1; ++t) g.out[(int64_t)t * g.H * g.dv + h * g.dv + j] = 0.f;
+    if (part == 0)
+      for (int t = r0; t < r1; ++t)
+        for (int c = 0; c < kCols; ++c)
+          if (j0 + c < g.dv) g.out[(int64_t)t * g.H * g.dv + h * g.dv + j0 + c] = 0.f;
     return;
   }
   const int i0 = part * kRows;
-  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv + (col_ok ? j : 0)) * g.dk + i0;
+  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv) * g.dk + i0;  // + column * dk
   const bool fresh = g.pos[r0] == 0;
   const bool vec = g.dk % 4 == 0 && i0 + kRows <= g.dk;
-  float S[kRows];
+  float S[kCols][kRows];
 #pragma unroll
-  for (int q = 0; q < kRows; ++q) S[q] = 0.f;
-  if (!fresh && col_ok) {
+  for (int c = 0; c < kCols; ++c) {
+#pragma unroll
+    for (int q = 0; q < kRows; ++q) S[c][q] = 0.f;
+    if (fresh || j0 + c >= g.dv) continue;
+    const float* spc = sp + (int64_t)(j0 + c) * g.dk;
     if (vec) {
 #pragma unroll
       for (int q = 0; q < kRows; q += 4) {
-        const f32x4 x = *reinterpret_cast<const f32x4*>(sp + q);
-        S[q] = x[0], S[q + 1] = x[1], S[q + 2] = x[2], S[q + 3] = x[3];
+        const f32x4 x = *reinterpret_cast<const f32x4*>(spc + q);
+        S[c][q] = x[0], S[c][q + 1] = x[1], S[c][q + 2] = x[2], S[c][q + 3] = x[3];
       }
     } else {
 #pragma unroll
       for (int q = 0; q < kRows; ++q)
-        if (i0 + q < g.dk) S[q] = sp[q];
+        if (i0 + q < g.dk) S[c][q] = spc[q];
     }
   }
   const T* pr = (const T*)g.r + (int64_t)h * g.dk;
   const T* pk = (const T*)g.k + (int64_t)h * g.dk;
   const T* pa = (const T*)g.a + (int64_t)h * g.dk;
   const T* pw = (const T*)g.w + (int64_t)h * g.dk;
-  const T* pv = (const T*)g.v + (int64_t)h * g.dv + blockIdx.z * kCols;
+  const T* pv = (const T*)g.v + (int64_t)h * g.dv + blockIdx.z * kWgCols;
   float fr[kE], fk[kE], fa[kE], fw[kE], fv[kEv];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < kE; ++e) {
-      const int idx = tid + e * kDThreads, tt = idx / kDkp, ch = idx % kDkp;
+      const int idx = tid + e * NT, tt = idx / kDkp, ch = idx % kDkp;
       const bool ok = idx < kTok * kDkp && t0 + tt < n && ch < g.dk;
       const int64_t row = r0 + t0 + tt;
       fr[e] = ok ? ldf<T>(pr, row * g.rs + ch) : 0.f;
@@ -121,18 +141,20 @@ __global__ void __launch_bounds__(kDThreads) delta_rule_kernel(DeltaArgs g) {
     }
 #pragma unroll
     for (int e = 0; e < kEv; ++e) {
-      const int idx = tid + e * kDThreads, tt = idx / kCols, cc = idx % kCols;
-      const bool ok = idx < kTok * kCols && t0 + tt < n && blockIdx.z * kCols + cc < g.dv;
+      const int idx = tid + e * NT, tt = idx / kWgCols, cc = idx % kWgCols;
+      const bool ok = idx < kTok * kWgCols && t0 + tt < n && blockIdx.z * kWgCols + cc < g.dv;
       fv[e] = ok ? ldf<T>(pv, (int64_t)(r0 + t0 + tt) * g.vs + cc) : 0.f;
     }
   };
   fetch(0);
   const int lane = tid & 63, wv = tid >> 6;
+  float* outp = g.out + (int64_t)r0 * g.H * g.dv + h * g.dv + j0;
+  const bool out4 = g.dv % 4 == 0 && j0 + kCols <= g.dv;
   for (int t0 = 0; t0 < n; t0 += kTok) {
     __syncthreads();  // the previous block's tokens are consumed
 #pragma unroll
     for (int e = 0; e < kE; ++e) {
-      const int idx = tid + e * kDThreads, tt = idx / kDkp, ch = idx % kDkp;
+      const int idx = tid + e * NT, tt = idx / kDkp, ch = idx % kDkp;
       if (idx < kTok * kDkp) {
         sr[tt][ch] = fr[e];
         sk[tt][ch] = fk[e];
@@ -143,13 +165,13 @@ __global__ void __launch_bounds__(kDThreads) delta_rule_kernel(DeltaArgs g) {
     }
 #pragma unroll
     for (int e = 0; e < kEv; ++e) {
-      const int idx = tid + e * kDThreads;
-      if (idx < kTok * kCols) sv[idx / kCols][idx % kCols] = fv[e];
+      const int idx = tid + e * NT;
+      if (idx < kTok * kWgCols) sv[idx / kWgCols][idx % kWgCols] = fv[e];
     }
     __syncthreads();
     if (t0 + kTok < n) fetch(t0 + kTok);
-    // unit keys: one wave per token, kTok / 4 tokens each
-    for (int tt = wv; tt < kTok; tt += kDThreads / 64) {
+    // unit keys: a wave per token in turn
+    for (int tt = wv; tt < kTok; tt += NT / 64) {
       float ss = 0.f;
       for (int ch = lane; ch < kDkp; ch += 64) ss += sk[tt][ch] * sk[tt][ch];
       const float inv = rsqrtf(wave_reduce_sum(ss) + g.key_eps);
@@ -162,67 +184,93 @@ __global__ void __launch_bounds__(kDThreads) delta_rule_kernel(DeltaArgs g) {
     __syncthreads();
     const int nt = n - t0 < kTok ? n - t0 : kTok;
     for (int tt = 0; tt < nt; ++tt) {
-      float u[kRows], x[kRows];
+      float x[kRows], y[kRows], us[kCols], o_[kCols];
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(u + q) = *reinterpret_cast<const f32x4*>(&su[tt][i0 + q]);
-      float us = 0.f;
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&su[tt][i0 + q]);
 #pragma unroll
-      for (int q = 0; q < kRows; ++q) us += u[q] * S[q];
+      for (int c = 0; c < kCols; ++c) {
+        float a_ = 0.f;
 #pragma unroll
-      for (int o = 1; o < R; o <<= 1) us += __shfl_xor(us, o, 64);
-      const float vj = sv[tt][c];
+        for (int q = 0; q < kRows; ++q) a_ += x[q] * S[c][q];
+        us[c] = group_sum<R>(a_);
+      }
+      const f32x4 vj = *reinterpret_cast<const f32x4*>(&sv[tt][grp * kCols]);
 #pragma unroll
       for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sw[tt][i0 + q]);
 #pragma unroll
-      for (int q = 0; q < kRows; ++q) S[q] *= x[q];
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sa[tt][i0 + q]);
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sa[tt][i0 + q]);
+      for (int c = 0; c < kCols; ++c)
 #pragma unroll
-      for (int q = 0; q < kRows; ++q) S[q] -= x[q] * us;
+        for (int q = 0; q < kRows; ++q) S[c][q] = S[c][q] * x[q] - y[q] * us[c];
 #pragma unroll
       for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sk[tt][i0 + q]);
 #pragma unroll
-      for (int q = 0; q < kRows; ++q) S[q] += x[q] * vj;
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sr[tt][i0 + q]);
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sr[tt][i0 + q]);
-      float o_ = 0.f;
+      for (int c = 0; c < kCols; ++c) {
+        float a_ = 0.f;
 #pragma unroll
-      for (int q = 0; q < kRows; ++q) o_ += x[q] * S[q];
+        for (int q = 0; q < kRows; ++q) {
+          S[c][q] += x[q] * vj[c];
+          a_ += y[q] * S[c][q];
+        }
+        o_[c] = group_sum<R>(a_);
+      }
+      if (part == 0) {
+        float* op = outp + (int64_t)(t0 + tt) * g.H * g.dv;
+        if (out4) {
+          *reinterpret_cast<f32x4*>(op) = f32x4{o_[0], o_[1], o_[2], o_[3]};
+        } else {
 #pragma unroll
-      for (int o = 1; o < R; o <<= 1) o_ += __shfl_xor(o_, o, 64);
-      if (part == 0 && col_ok) g.out[(int64_t)(r0 + t0 + tt) * g.H * g.dv + h * g.dv + j] = o_;
+          for (int c = 0; c < kCols; ++c)
+            if (j0 + c < g.dv) op[c] = o_[c];
+        }
+      }
     }
   }
-  if (col_ok) {
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    if (j0 + c >= g.dv) continue;
+    float* spc = sp + (int64_t)(j0 + c) * g.dk;
     if (vec) {
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(sp + q) = f32x4{S[q], S[q + 1], S[q + 2], S[q + 3]};
+      for (int q = 0; q < kRows; q += 4)
+        *reinterpret_cast<f32x4*>(spc + q) = f32x4{S[c][q], S[c][q + 1], S[c][q + 2], S[c][q + 3]};
     } else {
 #pragma unroll
       for (int q = 0; q < kRows; ++q)
-        if (i0 + q < g.dk) sp[q] = S[q];
+        if (i0 + q < g.dk) spc[q] = S[c][q];
     }
   }
 }
 
+// NT threads per workgroup: enough for all columns of a head, at most 256
 template <typename T, int R>
 void launch_delta(const DeltaArgs& g, int n_seq, hipStream_t st) {
-  const int cols = kDThreads / R;
-  hipLaunchKernelGGL((delta_rule_kernel<T, R>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(kDThreads), 0, st, g);
+  const int need = R * ((g.dv + kCols - 1) / kCols);
+  if (need <= 64) {
+    hipLaunchKernelGGL((delta_rule_kernel<T, R, 64>), dim3(n_seq, g.H, 1), dim3(64), 0, st, g);
+  } else if (need <= 128) {
+    hipLaunchKernelGGL((delta_rule_kernel<T, R, 128>), dim3(n_seq, g.H, 1), dim3(128), 0, st, g);
+  } else {
+    const int cols = 256 / R * kCols;
+    hipLaunchKernelGGL((delta_rule_kernel<T, R, 256>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(256), 0, st, g);
+  }
 }
 
 // ---------------------------------------------------------------------------
 // Short causal convolution over time on the leading C = n_q d + n_k (d + dv)
 // columns of a fused projection, then rotary positions on the first 2 * half
 // columns of every q and k head (column i paired with i + half), q to its own
-// tensor, k and v into the paged caches.  y_t = sum_j cw[c][j] u_(t - taps + 1 + j);
+// tensor, k and v into the paged caches.  y_t = sum_j cw[j][c] u_(t - taps + 1 + j);
 // u at positions before the step's first row of the sequence comes from the
 // sequence's tail state [taps - 1, C], and is zero before position 0.
 struct ConvArgs {
   void* q_out;  // [T, n_q * d]
   const void* x;
   int64_t xs;
-  const float* cw;  // [C, taps]
+  const float* cw;  // [taps, C] (tap-major: a run of channels shares a load)
   int taps;
   const void* tail;  // [slots, taps - 1, C]
   int n_slots;
@@ -259,7 +307,7 @@ __global__ void __launch_bounds__(256) conv_rope_cache_kernel(ConvArgs g) {
       float u = 0.f;
       if (qp >= p0) u = ldf<T>(x, (int64_t)(r0 + (qp - p0)) * g.xs + c);
       else if (qp >= 0) u = ldf<T>(tail, (qp - p0 + m) * C + c);
-      y += g.cw[(int64_t)c * g.taps + jj] * u;
+      y += g.cw[(int64_t)jj * C + c] * u;
     }
     return y;
   };
@@ -280,6 +328,96 @@ __global__ void __launch_bounds__(256) conv_rope_cache_kernel(ConvArgs g) {
       else if (kvs >= 0 && live) stf<T>((T*)g.kc, kvs * (g.n_k * g.d) + (c - g.n_q * g.d), y);
     } else if (kvs >= 0 && live) {
       stf<T>((T*)g.vc, kvs * (g.n_k * g.dv) + (c - qk), y);
+    }
+  }
+}
+
+// The same on V consecutive channels per thread with 16-byte loads and stores (V = 8 bf16 or
+// 4 fp32): a thread takes a run of the low rotary half together with its partner run of the
+// high half, so every channel is convolved once and every angle evaluated once.  Needs d, dv,
+// half, the row stride and the cache widths to be multiples of V, and 16-byte aligned bases.
+template <typename T, int V> struct VecIO;
+template <> struct VecIO<bf16_t, 8> {
+  __device__ static __forceinline__ void ld(const bf16_t* p, float* o) {
+    const u16x8 a = *reinterpret_cast<const u16x8*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[2 * i] = bf16lo(a.w[i]), o[2 * i + 1] = bf16hi(a.w[i]);
+  }
+  __device__ static __forceinline__ void st(bf16_t* p, const float* v) {
+    u16x8 a;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a.w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+    *reinterpret_cast<u16x8*>(p) = a;
+  }
+};
+template <> struct VecIO<float, 4> {
+  __device__ static __forceinline__ void ld(const float* p, float* o) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    o[0] = a[0], o[1] = a[1], o[2] = a[2], o[3] = a[3];
+  }
+  __device__ static __forceinline__ void st(float* p, const float* v) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  }
+};
+
+template <typename T, int V>
+__global__ void __launch_bounds__(256) conv_rope_cache_vec_kernel(ConvArgs g) {
+  const int t = blockIdx.x;
+  const int C = g.n_q * g.d + g.n_k * (g.d + g.dv);
+  const int s = g.row_seq ? g.row_seq[t] : t;
+  const bool seq_ok = s >= 0 && s < g.n_seq;
+  const int r0 = !seq_ok ? t : (g.seq_rows ? g.seq_rows[s] : t);
+  const int slot = seq_ok ? g.slots[s] : -1;
+  const bool live = slot >= 0 && slot < g.n_slots && r0 >= 0 && r0 <= t;
+  const int64_t p = g.pos[t];
+  const int64_t p0 = p - (t - r0);
+  const int m = g.taps - 1;
+  const T* x = (const T*)g.x;
+  const T* tail = (const T*)g.tail + (int64_t)(live ? slot : 0) * m * C;
+  auto conv = [&](int c, float* y) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) y[i] = 0.f;
+    if (!live) return;
+    for (int jj = 0; jj < g.taps; ++jj) {
+      const int64_t qp = p - m + jj;
+      if (qp < 0) continue;
+      float u[V], w[V];
+      if (qp >= p0) VecIO<T, V>::ld(x + (int64_t)(r0 + (qp - p0)) * g.xs + c, u);
+      else VecIO<T, V>::ld(tail + (qp - p0 + m) * C + c, u);
+      const float* wp = g.cw + (int64_t)jj * C + c;
+#pragma unroll
+      for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4*>(w + i) = *reinterpret_cast<const f32x4*>(wp + i);
+#pragma unroll
+      for (int i = 0; i < V; ++i) y[i] += w[i] * u[i];
+    }
+  };
+  const int qk = (g.n_q + g.n_k) * g.d, nq = g.n_q * g.d;
+  const int64_t kvs = live ? g.kv_slots[t] : -1;
+  auto put = [&](int c, const float* y) {
+    if (c < nq) VecIO<T, V>::st((T*)g.q_out + (int64_t)t * nq + c, y);
+    else if (kvs < 0) return;
+    else if (c < qk) VecIO<T, V>::st((T*)g.kc + kvs * (g.n_k * g.d) + (c - nq), y);
+    else VecIO<T, V>::st((T*)g.vc + kvs * (g.n_k * g.dv) + (c - qk), y);
+  };
+  for (int c = threadIdx.x * V; c < C; c += blockDim.x * V) {
+    const int e = c < qk ? c % g.d : 2 * g.half;
+    if (e >= g.half && e < 2 * g.half) continue;  // the high half rides with its low partner
+    float y[V];
+    conv(c, y);
+    if (e < g.half) {
+      float z[V], lo[V], hi[V];
+      conv(c + g.half, z);
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        float sn, cs;
+        sincosf((float)p * g.inv_freq[e + i], &sn, &cs);
+        lo[i] = y[i] * cs - z[i] * sn;
+        hi[i] = z[i] * cs + y[i] * sn;
+      }
+      put(c, lo);
+      put(c + g.half, hi);
+    } else {
+      put(c, y);
     }
   }
 }
@@ -378,7 +516,13 @@ int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw,
   if ((row_seq == nullptr) != (seq_rows == nullptr) || (!row_seq && n_seq != T_)) return 3;
   ConvArgs g{q_out, x, xs, cw, taps, tail, n_slots, pos, kv_slots, row_seq, seq_rows, slots, n_seq, T_,
              n_q, n_k, d, dv, inv_freq, half, kc, vc};
-  DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), 0, st, g));
+  const int V = f32 ? 4 : 8, esz = f32 ? 4 : 2;
+  auto al = [&](const void* ptr) { return (uintptr_t)ptr % 16 == 0; };
+  const bool vec = d % V == 0 && dv % V == 0 && half % V == 0 && xs % V == 0 && al(x) && al(q_out) && al(tail) &&
+                   al(kc) && al(vc) && al(cw) && ((n_q * d + n_k * (d + dv)) * esz) % 16 == 0;
+  if (vec && f32) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<float, 4>), dim3(T_), dim3(256), 0, st, g);
+  else if (vec) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<bf16_t, 8>), dim3(T_), dim3(256), 0, st, g);
+  else { DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), 0, st, g)); }
   DX_CHECK_LAUNCH();
   return 0;
 }

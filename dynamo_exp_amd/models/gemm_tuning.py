@@ -54,11 +54,15 @@ def tune_small_m(groups: list[list[torch.Tensor]], sizes, plan: dict, tuned: set
                 lib = _timed(lambda: [torch.matmul(x, w.t()) for w in ws], reps) / len(ws)
                 best = None
                 for cfg in cfgs:
-                    t = _timed(lambda: [ops.skinny_linear(x, w, cfg) for w in ws], reps) / len(ws)
+                    try:
+                        t = _timed(lambda: [ops.skinny_linear(x, w, cfg) for w in ws], reps) / len(ws)
+                    except ValueError:  # a launch configuration that does not divide this N or K
+                        continue
                     if best is None or t < best[0]:
                         best = (t, cfg)
-                row.update(lib_us=round(lib, 2), best_us=round(best[0], 2), cfg=best[1])
-                if best[0] < lib * (1 - min_gain):
+                row.update(lib_us=round(lib, 2), best_us=round(best[0], 2) if best else None,
+                           cfg=best[1] if best else None)
+                if best is not None and best[0] < lib * (1 - min_gain):
                     for w in (ws[0], ws[-1]):
                         want = torch.matmul(x, w.t()).float()
                         got = ops.skinny_linear(x, w, best[1]).float()

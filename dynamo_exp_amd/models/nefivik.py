@@ -50,6 +50,8 @@ from .llama import AttnMeta, TPGroup
 
 MIXERS = ("general_delta", "attention")
 EXPERT_ALPHA = 1.702  # the experts' gate is g * sigmoid(EXPERT_ALPHA * g)
+IN_PAD = 64  # fused in-projections end in narrow sections (a gate per head, the decay's inner width): their
+#              row count is padded with zero rows to a multiple of this, the GEMM kernels' column tile
 
 
 class NefivikForCausalLM:
@@ -114,8 +116,12 @@ class NefivikForCausalLM:
         library (bf16 on the GPU; models/gemm_tuning.py)."""
         if self.device.type != "cuda" or self.dtype != torch.bfloat16 or not self.layers:
             return []
-        groups = [[L[n] for L in self.layers if L.get(n) is not None] for n in self.LINEARS]
-        return tune_small_m([g for g in groups if g], sizes, self.gemm_plan, self.gemm_tuned, **kw)
+        groups: dict = {}  # layers of different mixers have in-projections of different shapes
+        for n in self.LINEARS:
+            for L in self.layers:
+                if L.get(n) is not None:
+                    groups.setdefault((n, tuple(L[n].shape)), []).append(L[n])
+        return tune_small_m(list(groups.values()), sizes, self.gemm_plan, self.gemm_tuned, **kw)
 
     def _mm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         return planned_mm(self.gemm_plan, x, w)
@@ -275,8 +281,10 @@ class NefivikForCausalLM:
         convolution taps and rotary frequencies in fp32."""
         cfg, dev, dt = self.cfg, self.device, self.dtype
 
-        def act(*names):  # (fused) projection weight
+        def act(*names, pad: int = 0):  # (fused) projection weight; pad: zero rows up to a multiple of it
             t = torch.cat([sd[n] for n in names], 0) if len(names) > 1 else sd[names[0]]
+            if pad and t.shape[0] % pad:
+                t = torch.cat([t, t.new_zeros((pad - t.shape[0] % pad, t.shape[1]))], 0)
             return t.to(dev, dt).contiguous()
 
         def f32(t):
@@ -289,16 +297,17 @@ class NefivikForCausalLM:
             out = dict(m=m, type=L["type"], mlp=mlp, norm1=f32(sd[q + "norm1"]), norm1b=f32(sd[q + "norm1b"]),
                        rg1_b=f32(sd[q + "rg1.b"]), w_o=act(p + "o"))
             if L["type"] == "general_delta":
-                out.update(w_in=act(p + "r", p + "k", p + "v", p + "g", p + "a", q + "rg1", p + "w1"),
+                out.update(w_in=act(p + "r", p + "k", p + "v", p + "g", p + "a", q + "rg1", p + "w1", pad=IN_PAD),
                            w_w2=act(p + "w2"), a_b=f32(sd[p + "a.b"]), w0=f32(sd[p + "w0"]), hnorm=f32(sd[p + "norm"]),
                            lora=sd[p + "w1"].shape[0])
             else:
                 own = m.get("kv_from") is None
                 names = [p + "q"] + ([p + "k", p + "v"] if own else [])
-                out.update(w_in=act(*names, q + "rg1", p + "g"), pb=f32(sd[p + "pb"]), own=own)
+                out.update(w_in=act(*names, q + "rg1", p + "g", pad=IN_PAD), pb=f32(sd[p + "pb"]), own=own)
                 taps = int(m.get("conv") or 0)
-                out["conv_w"] = f32(torch.cat([sd[n + ".conv"] for n in names], 0)) if taps else \
-                    torch.ones((self._conv_channels(m), 1), dtype=torch.float32, device=dev)
+                # tap-major [taps, C]: a run of neighbouring channels shares one load in the kernel
+                out["conv_w"] = f32(torch.cat([sd[n + ".conv"] for n in names], 0).t()) if taps else \
+                    torch.ones((1, self._conv_channels(m)), dtype=torch.float32, device=dev)
                 rot = m.get("rot")
                 out["inv_freq"] = rc.rotary_frequencies(rot["dims"], rot["base"], rot.get("scaling")).to(dev) \
                     if rot and rot.get("dims") else None
@@ -348,7 +357,7 @@ class NefivikForCausalLM:
         m, T, W = L["m"], h.shape[0], self.cfg.hidden_size
         H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         p = self._mm(h, L["w_in"])  # [q | k | v | rg1 | g]  (k, v only with keys of its own)
-        C = L["conv_w"].shape[0]
+        C = L["conv_w"].shape[1]
         q = rc.conv_rope_cache(p, L["conv_w"], cstate, meta.positions, meta.slot_mapping,
                                meta.row_seq if meta.is_prefill else None, meta.seq_rows, meta.state_slots, H,
                                G if L["own"] else 0, d, dv, L["inv_freq"], kc if L["own"] else None,

@@ -64,7 +64,8 @@ def conv_rope_cache(x: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Ten
                     kc: torch.Tensor | None, vc: torch.Tensor | None) -> torch.Tensor:
     """Per row of a fused projection x = [q (n_q d) | k (n_k d) | v (n_k dv) | ...]:
     every channel c of the C = n_q d + n_k (d + dv) leading columns is
-    convolved over time, y_t = sum_j conv_w[c, j] u_(t - taps + 1 + j), where u
+    convolved over time, y_t = sum_j conv_w[j, c] u_(t - taps + 1 + j) (conv_w
+    [taps, C] fp32, tap-major: the transpose of a checkpoint's [C, taps]), where u
     at a position before the step's first row of the sequence comes from
     conv_state [slots, taps - 1, C] (the last taps - 1 projected rows the
     sequence had before this step) and is zero before position 0.  Then the
@@ -75,7 +76,7 @@ def conv_rope_cache(x: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Ten
     no caches, a layer that reads another layer's).  conv_state is not changed
     (conv_state_update does that, after this)."""
     T = x.shape[0]
-    C, taps = conv_w.shape
+    taps, C = conv_w.shape
     n_seq = state_slots.numel()
     _fp32_param(conv_w, "conv_w")
     _fp32_param(inv_freq, "inv_freq")
@@ -103,7 +104,7 @@ def conv_rope_cache(x: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Ten
                     hist[m] = 0.0
             u = torch.cat([hist, x[r0:r1, :C].float()], 0)
             for j in range(taps):
-                y[r0:r1] += u[j:j + r1 - r0] * conv_w[:, j]
+                y[r0:r1] += u[j:j + r1 - r0] * conv_w[j]
         qk = y[:, : (n_q + n_k) * d].reshape(T, n_q + n_k, d)
         if half:
             ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]

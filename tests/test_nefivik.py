@@ -234,14 +234,15 @@ def test_delta_rule_removes_and_decays(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("taps,half,n_k", [(3, 4, 2), (1, 0, 2), (5, 10, 0), (2, 3, 1)])
-def test_conv_rope_cache_alone(device, taps, half, n_k):
+@pytest.mark.parametrize("taps,half,n_k,d,dv", [(3, 4, 2, 20, 6), (1, 0, 2, 20, 6), (5, 10, 0, 20, 6), (2, 3, 1, 20, 6),
+                                               (4, 8, 2, 32, 16), (3, 16, 1, 32, 8), (2, 0, 2, 16, 24)])
+def test_conv_rope_cache_alone(device, taps, half, n_k, d, dv):
     """Short convolution, rotation and cache write of two sequences, whole and in portions down to
     one row (shorter than the taps), slots reused with garbage in them, against the oracle."""
     torch.manual_seed(taps)
-    n_q, d, dv, T, bs = 3, 20, 6, 23, 4
+    n_q, T, bs = 3, 23, 4
     C = n_q * d + n_k * (d + dv)
-    x = torch.randn(2, T, C + 5)
+    x = torch.randn(2, T, C + (5 if d % 8 else 8))  # (the wide shapes keep rows 16-byte aligned: the vector kernel)
     cw = torch.randn(C, taps)
     rot = {"base": 50.0, "dims": 2 * half, "scaling": {"factor": 4.0, "low": 1.0, "high": 3.0, "original": 16}}
     inv = rc.rotary_frequencies(2 * half, 50.0, rot["scaling"]) if half else None
@@ -267,7 +268,7 @@ def test_conv_rope_cache_alone(device, taps, half, n_k):
         pos, row_seq, seq_rows, slots = step_meta(device, cuts, [2 if s == 0 else 0 for s in live])
         xs = torch.cat([x[s, p:p + n] for s, (p, n) in zip(live, cuts)]).to(device)
         kvs = torch.cat([slot_of(s, torch.arange(p, p + n)) for s, (p, n) in zip(live, cuts)]).to(device)
-        q = rc.conv_rope_cache(xs, d_(cw), tail, pos, kvs, row_seq, seq_rows, slots, n_q, n_k, d, dv, d_(inv), kc, vc)
+        q = rc.conv_rope_cache(xs, d_(cw.t().contiguous()), tail, pos, kvs, row_seq, seq_rows, slots, n_q, n_k, d, dv, d_(inv), kc, vc)
         rc.conv_state_update(xs, tail, pos, seq_rows, slots)
         for i, (s, (p, n)) in enumerate(zip(live, cuts)):
             got[s].append(q[int(seq_rows[i]):int(seq_rows[i]) + n].cpu())
