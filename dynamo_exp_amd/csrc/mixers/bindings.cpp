@@ -24,7 +24,7 @@ int dxm_residual_step(float*, const void*, int64_t, const void*, int64_t, const 
                       int, hipStream_t);
 int dxm_act_mul(void*, const void*, int64_t, const void*, int64_t, int, int, int64_t, int, float, float, int,
                 hipStream_t);
-int dxm_delta_rule(float*, float*, int, const void*, int64_t, const void*, int64_t, const void*, int64_t, const void*,
+int dxm_delta_rule(float*, float*, int, float*, const void*, int64_t, const void*, int64_t, const void*, int64_t, const void*,
                    int64_t, const void*, int64_t, const float*, const float*, float, float, const int64_t*, const int*,
                    const int*, int, int, int, int, int, int, hipStream_t);
 int dxm_conv_rope_cache(void*, const void*, int64_t, const float*, int, const void*, int, const int64_t*,
@@ -97,10 +97,10 @@ PYBIND11_MODULE(_C_mixers, m) {
                         S(st)),
           "moe_route");
   });
-  m.def("delta_rule", [](u out, u state, int n_slots, u r, int64_t rs, u k, int64_t ks, u v, int64_t vs, u a,
+  m.def("delta_rule", [](u out, u state, int n_slots, u prep, u r, int64_t rs, u k, int64_t ks, u v, int64_t vs, u a,
                          int64_t as, u w, int64_t ws, u ab, u wb, float decay_scale, float key_eps, u pos, u seq_rows,
                          u slots, int n_seq, int T, int H, int dk, int dv, int f32, u st) {
-    check(dxm_delta_rule(F(out), F(state), n_slots, P(r), rs, P(k), ks, P(v), vs, P(a), as, P(w), ws, F(ab), F(wb),
+    check(dxm_delta_rule(F(out), F(state), n_slots, F(prep), P(r), rs, P(k), ks, P(v), vs, P(a), as, P(w), ws, F(ab), F(wb),
                          decay_scale, key_eps, reinterpret_cast<const int64_t*>(pos),
                          reinterpret_cast<const int*>(seq_rows), reinterpret_cast<const int*>(slots), n_seq, T, H, dk,
                          dv, f32, S(st)),

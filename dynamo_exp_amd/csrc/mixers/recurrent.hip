@@ -30,28 +30,29 @@ __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-
 //     S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,   o_t = S_t^T r_t
 // with w_t = exp(-decay_scale * sigmoid(wl_t + w_bias)), a_t = sigmoid(al_t + a_bias),
 // u_t = k_t / sqrt(sum(k_t^2) + key_eps).  Columns of S are independent, so a
-// thread owns a tile of kRows consecutive rows x kCols consecutive columns in
-// registers (every row vector it reads from LDS serves kCols columns), R
+// thread owns a tile of kRows consecutive rows x CT consecutive columns in
+// registers (every row vector it reads from LDS serves CT columns), R
 // neighbouring lanes share the columns and join their partial dot products by
 // DPP lane exchanges (no LDS traffic), and a workgroup of NT threads owns
-// NT / R * kCols columns of one (sequence, head).  The state tensor is stored
-// column-major per head ([slots, H, dv, dk]) so that a wave's state traffic is
-// contiguous runs.  Tokens are staged through LDS kTok at a time: raw r, k, a,
-// w, v rows are fetched into registers one block ahead (their latency hides
-// behind the current block's recurrence), committed, transformed in place
-// (sums of squares by wave reductions), and consumed token by token.
+// NT / R * CT columns of one (sequence, head).  CT is 4 where the launch has
+// waves to fill the chip and 2 where it has not (a few long prompts): the
+// recurrence is bound by instruction issue, so it wants every SIMD busy.  The
+// state tensor is stored column-major per head ([slots, H, dv, dk]) so that a
+// wave's state traffic is contiguous runs.  What the recurrence needs per
+// token and key channel beside r and k -- the unit key u, the decay w and
+// a * u -- is computed for all rows at once by delta_prep_kernel (fp32, [T, H,
+// 3, dk]): it is elementwise work and would otherwise sit in the sequential
+// chain.  Tokens are staged through LDS kTok at a time, fetched into registers
+// one block ahead (the latency hides behind the current block's recurrence).
 constexpr int kRows = 16;  // state rows per thread
-constexpr int kCols = 4;   // state columns per thread
 constexpr int kTok = 8;    // tokens per staged block
 
 struct DeltaArgs {
   float* out;    // [T, H * dv]
   float* state;  // [slots, H, dv, dk]
-  const void *r, *k, *v, *a, *w;
-  int64_t rs, ks, vs, as, ws;  // row strides (elements)
-  const float* a_bias;         // [H * dk] or null
-  const float* w_bias;
-  float decay_scale, key_eps;
+  const void *r, *k, *v;
+  int64_t rs, ks, vs;  // row strides (elements)
+  const float* prep;   // [T, H, 3, dk]: unit key, decay, removal rate * unit key
   const int64_t* pos;
   const int* seq_rows;  // null: row i is sequence i
   const int* slots;
@@ -72,8 +73,36 @@ template <int R> __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <typename T, int R, int NT>
+// one wave per (row, head): u = k / sqrt(sum k^2 + key_eps), w = exp(-decay_scale sigmoid(wl + w_bias)),
+// a u with a = sigmoid(al + a_bias)
+template <typename T>
+__global__ void __launch_bounds__(64) delta_prep_kernel(float* __restrict__ prep, const T* __restrict__ k, int64_t ks,
+                                                        const T* __restrict__ a, int64_t as, const T* __restrict__ w,
+                                                        int64_t ws, const float* __restrict__ a_bias,
+                                                        const float* __restrict__ w_bias, float decay_scale,
+                                                        float key_eps, int H, int dk) {
+  const int64_t v = blockIdx.x, row = v / H;
+  const int h = (int)(v - row * H), lane = threadIdx.x;
+  const T* kp = k + row * ks + (int64_t)h * dk;
+  float ss = 0.f;
+  for (int ch = lane; ch < dk; ch += 64) {
+    const float x = ldf<T>(kp, ch);
+    ss += x * x;
+  }
+  const float inv = rsqrtf(wave_reduce_sum(ss) + key_eps);
+  float* o = prep + v * 3 * dk;
+  for (int ch = lane; ch < dk; ch += 64) {
+    const float u = ldf<T>(kp, ch) * inv;
+    const float ab = a_bias ? a_bias[h * dk + ch] : 0.f, wb = w_bias ? w_bias[h * dk + ch] : 0.f;
+    o[ch] = u;
+    o[dk + ch] = expf(-decay_scale * sigmoidf_(ldf<T>(w, row * ws + (int64_t)h * dk + ch) + wb));
+    o[2 * dk + ch] = sigmoidf_(ldf<T>(a, row * as + (int64_t)h * dk + ch) + ab) * u;
+  }
+}
+
+template <typename T, int R, int NT, int CT>
 __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
+  constexpr int kCols = CT;
   constexpr int kGroups = NT / R;            // column tiles per workgroup
   constexpr int kWgCols = kGroups * kCols;   // columns per workgroup
   constexpr int kDkp = kRows * R;            // padded key width
@@ -99,10 +128,14 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
           if (j0 + c < g.dv) g.out[(int64_t)t * g.H * g.dv + h * g.dv + j0 + c] = 0.f;
     return;
   }
-  const int i0 = part * kRows;
-  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv) * g.dk + i0;  // + column * dk
+  // The thread's 16 rows are four quads, quad m at row (m * R + part) * 4: for one m the R lanes of a
+  // group read R consecutive 16-byte pieces of a row vector, so a wave's LDS read touches every bank once
+  // (16 consecutive rows per lane would put lanes 0, 2, 4, .. on the same banks).
+  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv) * g.dk;  // + column * dk + row
   const bool fresh = g.pos[r0] == 0;
-  const bool vec = g.dk % 4 == 0 && i0 + kRows <= g.dk;
+  int rq[kRows / 4];
+#pragma unroll
+  for (int m = 0; m < kRows / 4; ++m) rq[m] = (m * R + part) * 4;
   float S[kCols][kRows];
 #pragma unroll
   for (int c = 0; c < kCols; ++c) {
@@ -110,34 +143,35 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
     for (int q = 0; q < kRows; ++q) S[c][q] = 0.f;
     if (fresh || j0 + c >= g.dv) continue;
     const float* spc = sp + (int64_t)(j0 + c) * g.dk;
-    if (vec) {
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) {
-        const f32x4 x = *reinterpret_cast<const f32x4*>(spc + q);
-        S[c][q] = x[0], S[c][q + 1] = x[1], S[c][q + 2] = x[2], S[c][q + 3] = x[3];
+    for (int m = 0; m < kRows / 4; ++m) {
+      if (g.dk % 4 == 0 && rq[m] + 4 <= g.dk) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(spc + rq[m]);
+        S[c][4 * m] = x[0], S[c][4 * m + 1] = x[1], S[c][4 * m + 2] = x[2], S[c][4 * m + 3] = x[3];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (rq[m] + e < g.dk) S[c][4 * m + e] = spc[rq[m] + e];
       }
-    } else {
-#pragma unroll
-      for (int q = 0; q < kRows; ++q)
-        if (i0 + q < g.dk) S[c][q] = spc[q];
     }
   }
   const T* pr = (const T*)g.r + (int64_t)h * g.dk;
   const T* pk = (const T*)g.k + (int64_t)h * g.dk;
-  const T* pa = (const T*)g.a + (int64_t)h * g.dk;
-  const T* pw = (const T*)g.w + (int64_t)h * g.dk;
+  const float* pp = g.prep + (int64_t)h * 3 * g.dk;
   const T* pv = (const T*)g.v + (int64_t)h * g.dv + blockIdx.z * kWgCols;
-  float fr[kE], fk[kE], fa[kE], fw[kE], fv[kEv];
+  float fr[kE], fk[kE], fu[kE], fa[kE], fw[kE], fv[kEv];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int e = 0; e < kE; ++e) {
       const int idx = tid + e * NT, tt = idx / kDkp, ch = idx % kDkp;
       const bool ok = idx < kTok * kDkp && t0 + tt < n && ch < g.dk;
       const int64_t row = r0 + t0 + tt;
+      const float* pq = pp + row * g.H * 3 * g.dk + ch;
       fr[e] = ok ? ldf<T>(pr, row * g.rs + ch) : 0.f;
       fk[e] = ok ? ldf<T>(pk, row * g.ks + ch) : 0.f;
-      fa[e] = ok ? ldf<T>(pa, row * g.as + ch) : 0.f;
-      fw[e] = ok ? ldf<T>(pw, row * g.ws + ch) : 0.f;
+      fu[e] = ok ? pq[0] : 0.f;
+      fw[e] = ok ? pq[g.dk] : 0.f;
+      fa[e] = ok ? pq[2 * g.dk] : 0.f;
     }
 #pragma unroll
     for (int e = 0; e < kEv; ++e) {
@@ -147,7 +181,6 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
     }
   };
   fetch(0);
-  const int lane = tid & 63, wv = tid >> 6;
   float* outp = g.out + (int64_t)r0 * g.H * g.dv + h * g.dv + j0;
   const bool out4 = g.dv % 4 == 0 && j0 + kCols <= g.dv;
   for (int t0 = 0; t0 < n; t0 += kTok) {
@@ -158,9 +191,9 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
       if (idx < kTok * kDkp) {
         sr[tt][ch] = fr[e];
         sk[tt][ch] = fk[e];
-        const bool in = ch < g.dk;
-        sa[tt][ch] = in ? sigmoidf_(fa[e] + (g.a_bias ? g.a_bias[h * g.dk + ch] : 0.f)) : 0.f;
-        sw[tt][ch] = in ? expf(-g.decay_scale * sigmoidf_(fw[e] + (g.w_bias ? g.w_bias[h * g.dk + ch] : 0.f))) : 0.f;
+        su[tt][ch] = fu[e];
+        sw[tt][ch] = fw[e];
+        sa[tt][ch] = fa[e];
       }
     }
 #pragma unroll
@@ -170,23 +203,11 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
     }
     __syncthreads();
     if (t0 + kTok < n) fetch(t0 + kTok);
-    // unit keys: a wave per token in turn
-    for (int tt = wv; tt < kTok; tt += NT / 64) {
-      float ss = 0.f;
-      for (int ch = lane; ch < kDkp; ch += 64) ss += sk[tt][ch] * sk[tt][ch];
-      const float inv = rsqrtf(wave_reduce_sum(ss) + g.key_eps);
-      for (int ch = lane; ch < kDkp; ch += 64) {
-        const float u = sk[tt][ch] * inv;
-        su[tt][ch] = u;
-        sa[tt][ch] *= u;
-      }
-    }
-    __syncthreads();
     const int nt = n - t0 < kTok ? n - t0 : kTok;
     for (int tt = 0; tt < nt; ++tt) {
       float x[kRows], y[kRows], us[kCols], o_[kCols];
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&su[tt][i0 + q]);
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&su[tt][rq[q / 4]]);
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
         float a_ = 0.f;
@@ -194,19 +215,21 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
         for (int q = 0; q < kRows; ++q) a_ += x[q] * S[c][q];
         us[c] = group_sum<R>(a_);
       }
-      const f32x4 vj = *reinterpret_cast<const f32x4*>(&sv[tt][grp * kCols]);
+      float vj[kCols];
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sw[tt][i0 + q]);
+      for (int c = 0; c < kCols; ++c) vj[c] = sv[tt][grp * kCols + c];
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sa[tt][i0 + q]);
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sw[tt][rq[q / 4]]);
+#pragma unroll
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sa[tt][rq[q / 4]]);
 #pragma unroll
       for (int c = 0; c < kCols; ++c)
 #pragma unroll
         for (int q = 0; q < kRows; ++q) S[c][q] = S[c][q] * x[q] - y[q] * us[c];
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sk[tt][i0 + q]);
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sk[tt][rq[q / 4]]);
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sr[tt][i0 + q]);
+      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sr[tt][rq[q / 4]]);
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
         float a_ = 0.f;
@@ -219,9 +242,10 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
       }
       if (part == 0) {
         float* op = outp + (int64_t)(t0 + tt) * g.H * g.dv;
-        if (out4) {
-          *reinterpret_cast<f32x4*>(op) = f32x4{o_[0], o_[1], o_[2], o_[3]};
-        } else {
+        if constexpr (kCols == 4) {
+          if (out4) *reinterpret_cast<f32x4*>(op) = f32x4{o_[0], o_[1], o_[2], o_[3]};
+        }
+        if (kCols != 4 || !out4) {
 #pragma unroll
           for (int c = 0; c < kCols; ++c)
             if (j0 + c < g.dv) op[c] = o_[c];
@@ -233,30 +257,37 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
   for (int c = 0; c < kCols; ++c) {
     if (j0 + c >= g.dv) continue;
     float* spc = sp + (int64_t)(j0 + c) * g.dk;
-    if (vec) {
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4)
-        *reinterpret_cast<f32x4*>(spc + q) = f32x4{S[c][q], S[c][q + 1], S[c][q + 2], S[c][q + 3]};
-    } else {
+    for (int m = 0; m < kRows / 4; ++m) {
+      if (g.dk % 4 == 0 && rq[m] + 4 <= g.dk) {
+        *reinterpret_cast<f32x4*>(spc + rq[m]) = f32x4{S[c][4 * m], S[c][4 * m + 1], S[c][4 * m + 2], S[c][4 * m + 3]};
+      } else {
 #pragma unroll
-      for (int q = 0; q < kRows; ++q)
-        if (i0 + q < g.dk) spc[q] = S[c][q];
+        for (int e = 0; e < 4; ++e)
+          if (rq[m] + e < g.dk) spc[rq[m] + e] = S[c][4 * m + e];
+      }
     }
   }
 }
 
-// NT threads per workgroup: enough for all columns of a head, at most 256
+// NT threads per workgroup: 64 where that covers all columns of a head, else 256.  CT = 2 when
+// tiles of four columns would leave the launch under one wave per SIMD (1024 on the chip).
+template <typename T, int R, int CT>
+void launch_delta_ct(const DeltaArgs& g, int n_seq, hipStream_t st) {
+  const int need = R * ((g.dv + CT - 1) / CT);
+  if (need <= 64) {
+    hipLaunchKernelGGL((delta_rule_kernel<T, R, 64, CT>), dim3(n_seq, g.H, 1), dim3(64), 0, st, g);
+  } else {
+    const int cols = 256 / R * CT;
+    hipLaunchKernelGGL((delta_rule_kernel<T, R, 256, CT>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(256), 0,
+                       st, g);
+  }
+}
 template <typename T, int R>
 void launch_delta(const DeltaArgs& g, int n_seq, hipStream_t st) {
-  const int need = R * ((g.dv + kCols - 1) / kCols);
-  if (need <= 64) {
-    hipLaunchKernelGGL((delta_rule_kernel<T, R, 64>), dim3(n_seq, g.H, 1), dim3(64), 0, st, g);
-  } else if (need <= 128) {
-    hipLaunchKernelGGL((delta_rule_kernel<T, R, 128>), dim3(n_seq, g.H, 1), dim3(128), 0, st, g);
-  } else {
-    const int cols = 256 / R * kCols;
-    hipLaunchKernelGGL((delta_rule_kernel<T, R, 256>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(256), 0, st, g);
-  }
+  const int64_t waves4 = (int64_t)n_seq * g.H * ((R * ((g.dv + 3) / 4) + 63) / 64);
+  if (waves4 >= 1024) launch_delta_ct<T, R, 4>(g, n_seq, st);
+  else launch_delta_ct<T, R, 2>(g, n_seq, st);
 }
 
 // ---------------------------------------------------------------------------
@@ -311,6 +342,10 @@ __global__ void __launch_bounds__(256) conv_rope_cache_kernel(ConvArgs g) {
     }
     return y;
   };
+  // the row's angles: one cosine and sine per rotated pair, shared by all heads
+  extern __shared__ float cs_sn[];  // [half] cosines, [half] sines
+  for (int i = threadIdx.x; i < g.half; i += blockDim.x) sincosf((float)p * g.inv_freq[i], &cs_sn[g.half + i], &cs_sn[i]);
+  __syncthreads();
   const int qk = (g.n_q + g.n_k) * g.d;
   const int64_t kvs = g.kv_slots[t];
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
@@ -320,8 +355,7 @@ __global__ void __launch_bounds__(256) conv_rope_cache_kernel(ConvArgs g) {
       if (live && e < 2 * g.half) {
         const int i = e < g.half ? e : e - g.half;
         const float other = conv(e < g.half ? c + g.half : c - g.half);
-        float sn, cs;
-        sincosf((float)p * g.inv_freq[i], &sn, &cs);
+        const float cs = cs_sn[i], sn = cs_sn[g.half + i];
         y = e < g.half ? y * cs - other * sn : y * cs + other * sn;
       }
       if (c < g.n_q * g.d) stf<T>((T*)g.q_out, (int64_t)t * g.n_q * g.d + c, y);
@@ -391,6 +425,9 @@ __global__ void __launch_bounds__(256) conv_rope_cache_vec_kernel(ConvArgs g) {
       for (int i = 0; i < V; ++i) y[i] += w[i] * u[i];
     }
   };
+  extern __shared__ float cs_sn[];  // [half] cosines, [half] sines of the row's angles
+  for (int i = threadIdx.x; i < g.half; i += blockDim.x) sincosf((float)p * g.inv_freq[i], &cs_sn[g.half + i], &cs_sn[i]);
+  __syncthreads();
   const int qk = (g.n_q + g.n_k) * g.d, nq = g.n_q * g.d;
   const int64_t kvs = live ? g.kv_slots[t] : -1;
   auto put = [&](int c, const float* y) {
@@ -409,8 +446,7 @@ __global__ void __launch_bounds__(256) conv_rope_cache_vec_kernel(ConvArgs g) {
       conv(c + g.half, z);
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        float sn, cs;
-        sincosf((float)p * g.inv_freq[e + i], &sn, &cs);
+        const float cs = cs_sn[e + i], sn = cs_sn[g.half + e + i];
         lo[i] = y[i] * cs - z[i] * sn;
         hi[i] = z[i] * cs + y[i] * sn;
       }
@@ -483,22 +519,22 @@ __global__ void __launch_bounds__(64) head_norm_gate_kernel(T* __restrict__ out,
 
 extern "C" {
 
-int dxm_delta_rule(float* out, float* state, int n_slots, const void* r, int64_t rs, const void* k, int64_t ks,
-                   const void* v, int64_t vs, const void* a, int64_t as, const void* w, int64_t ws,
+int dxm_delta_rule(float* out, float* state, int n_slots, float* prep, const void* r, int64_t rs, const void* k,
+                   int64_t ks, const void* v, int64_t vs, const void* a, int64_t as, const void* w, int64_t ws,
                    const float* a_bias, const float* w_bias, float decay_scale, float key_eps, const int64_t* pos,
                    const int* seq_rows, const int* slots, int n_seq, int T_, int H, int dk, int dv, int f32,
                    hipStream_t st) {
   if (n_seq <= 0 || T_ <= 0) return 0;
-  if (H < 1 || dk < 1 || dv < 1 || n_slots < 1 || H > 65535 || n_seq > 0x7fffffff) return 1;
+  if (H < 1 || dk < 1 || dv < 1 || n_slots < 1 || H > 65535 || n_seq > 0x7fffffff || (int64_t)T_ * H > 0x7fffffff)
+    return 1;
   if (dk > kRows * 16) return 2;  // wider keys need more lanes per column than instantiated
-  if (!out || !state || !pos || !slots) return 3;
+  if (!out || !state || !pos || !slots || !prep) return 3;
   if (!seq_rows && n_seq != T_) return 4;
-  DeltaArgs g{out, state, r, k, v, a, w, rs, ks, vs, as, ws, a_bias, w_bias, decay_scale, key_eps,
-              pos, seq_rows, slots, n_slots, T_, H, dk, dv};
+  DISPATCH_T(f32, hipLaunchKernelGGL(delta_prep_kernel<T>, dim3((unsigned)(T_ * H)), dim3(64), 0, st, prep, (const T*)k,
+                                     ks, (const T*)a, as, (const T*)w, ws, a_bias, w_bias, decay_scale, key_eps, H, dk));
+  DeltaArgs g{out, state, r, k, v, rs, ks, vs, prep, pos, seq_rows, slots, n_slots, T_, H, dk, dv};
   const int need = (dk + kRows - 1) / kRows;
-  if (need <= 1) { DISPATCH_T(f32, (launch_delta<T, 1>(g, n_seq, st))); }
-  else if (need <= 2) { DISPATCH_T(f32, (launch_delta<T, 2>(g, n_seq, st))); }
-  else if (need <= 4) { DISPATCH_T(f32, (launch_delta<T, 4>(g, n_seq, st))); }
+  if (need <= 4) { DISPATCH_T(f32, (launch_delta<T, 4>(g, n_seq, st))); }
   else if (need <= 8) { DISPATCH_T(f32, (launch_delta<T, 8>(g, n_seq, st))); }
   else { DISPATCH_T(f32, (launch_delta<T, 16>(g, n_seq, st))); }
   DX_CHECK_LAUNCH();
@@ -510,7 +546,7 @@ int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw,
                         const int* seq_rows, const int* slots, int n_seq, int T_, int n_q, int n_k, int d, int dv,
                         const float* inv_freq, int half, void* kc, void* vc, int f32, hipStream_t st) {
   if (T_ <= 0) return 0;
-  if (taps < 1 || n_q < 0 || n_k < 0 || d < 1 || dv < 0 || half < 0 || 2 * half > d) return 1;
+  if (taps < 1 || n_q < 0 || n_k < 0 || d < 1 || dv < 0 || half < 0 || 2 * half > d || half > 4096) return 1;
   if ((half && !inv_freq) || (n_k && (!kc || !vc)) || (taps > 1 && !tail) || !cw || !pos || !kv_slots || !slots)
     return 2;
   if ((row_seq == nullptr) != (seq_rows == nullptr) || (!row_seq && n_seq != T_)) return 3;
@@ -520,9 +556,10 @@ int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw,
   auto al = [&](const void* ptr) { return (uintptr_t)ptr % 16 == 0; };
   const bool vec = d % V == 0 && dv % V == 0 && half % V == 0 && xs % V == 0 && al(x) && al(q_out) && al(tail) &&
                    al(kc) && al(vc) && al(cw) && ((n_q * d + n_k * (d + dv)) * esz) % 16 == 0;
-  if (vec && f32) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<float, 4>), dim3(T_), dim3(256), 0, st, g);
-  else if (vec) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<bf16_t, 8>), dim3(T_), dim3(256), 0, st, g);
-  else { DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), 0, st, g)); }
+  const size_t lds = (size_t)2 * half * sizeof(float);
+  if (vec && f32) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<float, 4>), dim3(T_), dim3(256), lds, st, g);
+  else if (vec) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<bf16_t, 8>), dim3(T_), dim3(256), lds, st, g);
+  else { DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), lds, st, g)); }
   DX_CHECK_LAUNCH();
   return 0;
 }

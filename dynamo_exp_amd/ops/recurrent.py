@@ -215,7 +215,9 @@ def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tenso
             state[sl] = S.transpose(1, 2)
         return out.view(T, H * dv)
     out = torch.empty((T, n_heads * dv), dtype=torch.float32, device=r.device)
-    _m().delta_rule(out.data_ptr(), state.data_ptr(), state.shape[0], r.data_ptr(), r.stride(0), k.data_ptr(),
+    # unit key, decay and removal rate * unit key of every row, formed by a pass of its own in front of the scan
+    prep = torch.empty((T, n_heads, 3, dk), dtype=torch.float32, device=r.device)
+    _m().delta_rule(out.data_ptr(), state.data_ptr(), state.shape[0], prep.data_ptr(), r.data_ptr(), r.stride(0), k.data_ptr(),
                     k.stride(0), v.data_ptr(), v.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0),
                     _ptr(a_bias), _ptr(w_bias), float(decay_scale), float(key_eps), positions.data_ptr(),
                     _ptr(seq_rows), state_slots.data_ptr(), n_seq, T, n_heads, dk, dv, _f32(r), _stream())
