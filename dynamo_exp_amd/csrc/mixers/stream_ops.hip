@@ -204,9 +204,20 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
       for (int i = 0; i < V; ++i) v[i] *= 1.f / (1.f + expf(-(gt[i] + (cgb ? gb[i] : 0.f))));
     }
   };
+  // (gated) addend: its chunks stay in registers between the mean square and the sum
+  float cv[kResChunks][V];
   if (c) {
     float ss = 0.f;
-    for (int e = threadIdx.x * V; e < W; e += kThreads * V) {
+#pragma unroll
+    for (int k = 0; k < kResChunks; ++k) {
+      const int e = (threadIdx.x + k * kThreads) * V;
+      if (e < W) {
+        load_c(e, cv[k]);
+#pragma unroll
+        for (int i = 0; i < V; ++i) ss += cv[k][i] * cv[k][i];
+      }
+    }
+    for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
       float v[V];
       load_c(e, v);
 #pragma unroll
@@ -237,10 +248,9 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
       }
       if (c) {
         float w[V];
-        load_c(e, t);
         ldv<float, V>(cw + e, w);
 #pragma unroll
-        for (int i = 0; i < V; ++i) r[k][i] += t[i] * rc * w[i];
+        for (int i = 0; i < V; ++i) r[k][i] += cv[k][i] * rc * w[i];
       }
       if (touch) stv<float, V>(x + e, r[k]);
       if (xc) stv<T, V>(xc + row * (int64_t)W + e, r[k]);
