@@ -317,7 +317,7 @@ def test_gated_residual_step(device, W):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("E,top,groups", [(12, 3, (3, 2)), (8, 2, (4, 2)), (6, 1, (6, 6)), (5, 2, None), (64, 4, (8, 3))])
+@pytest.mark.parametrize("E,top,groups", [(15, 3, (5, 2)), (8, 2, (4, 2)), (6, 1, (6, 6)), (5, 2, None), (64, 4, (8, 3))])
 def test_route_softmax_groups(device, E, top, groups):
     """Softmax scores, groups ranked by their best score.  One group is made to hold the two next-best
     experts after a clear winner elsewhere: ranked by the sum of two it would win, by its best it loses."""
@@ -341,8 +341,8 @@ def test_route_softmax_groups(device, E, top, groups):
     assert torch.equal(idx.cpu().long().sort(-1).values, idx_w.sort(-1).values)
     assert torch.allclose(w.cpu().double().sort(-1).values, w_w.sort(-1).values, atol=1e-6)
     assert float(w.sum(-1).max()) <= 1.0 + 1e-5  # softmax scores of the chosen, not renormalised
-    if groups == (3, 2) and top == 3:
-        assert not (idx.cpu() == 2 * (E // 3)).any() or groups[1] == 3
+    if groups and groups[0] >= 3 and groups[1] == 2 and E // groups[0] >= 2:
+        assert not (idx.cpu() == 2 * (E // groups[0])).any()  # the group of the best pair lost to the two best singles
 
 
 def paged(T, bs, n_blocks, width, device, dtype=torch.float32, seed=0):
@@ -443,7 +443,7 @@ def test_matrix_core_attention_sigmoid(size, dims):
 
 # ----------------------------------------------------------------- crafted: one key stands out
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("size,bs", [(40, 16), (17, 8), (1, 8), (200, 8)])
+@pytest.mark.parametrize("size,bs", [(44, 16), (17, 8), (1, 8), (200, 8)])
 def test_far_keys_window_edges(device, dtype, size, bs):
     """A cache of weak keys (weights near 0 through a negative head bias) in which one key matches
     the query strongly and carries a marked value: seen just inside the window, not just outside, at
