@@ -394,66 +394,110 @@ template <> struct VecIO<float, 4> {
   }
 };
 
+// A workgroup takes kConvRows consecutive rows of the step (they may belong to different
+// sequences); the taps loop is outermost, so a thread loads a tap's weights once for all its rows.
+constexpr int kConvRows = 4;
 template <typename T, int V>
-__global__ void __launch_bounds__(256) conv_rope_cache_vec_kernel(ConvArgs g) {
-  const int t = blockIdx.x;
+__global__ void __launch_bounds__(128) conv_rope_cache_vec_kernel(ConvArgs g) {
+  const int t0 = blockIdx.x * kConvRows;
   const int C = g.n_q * g.d + g.n_k * (g.d + g.dv);
-  const int s = g.row_seq ? g.row_seq[t] : t;
-  const bool seq_ok = s >= 0 && s < g.n_seq;
-  const int r0 = !seq_ok ? t : (g.seq_rows ? g.seq_rows[s] : t);
-  const int slot = seq_ok ? g.slots[s] : -1;
-  const bool live = slot >= 0 && slot < g.n_slots && r0 >= 0 && r0 <= t;
-  const int64_t p = g.pos[t];
-  const int64_t p0 = p - (t - r0);
   const int m = g.taps - 1;
   const T* x = (const T*)g.x;
-  const T* tail = (const T*)g.tail + (int64_t)(live ? slot : 0) * m * C;
-  auto conv = [&](int c, float* y) {
+  // per row: liveness, position, first position of its sequence in the step, first row, tail, cache slot
+  bool live[kConvRows];
+  int64_t p[kConvRows], p0[kConvRows], kvs[kConvRows];
+  int r0[kConvRows];
+  const T* tail[kConvRows];
 #pragma unroll
-    for (int i = 0; i < V; ++i) y[i] = 0.f;
-    if (!live) return;
+  for (int r = 0; r < kConvRows; ++r) {
+    const int t = t0 + r < g.T ? t0 + r : g.T - 1;
+    const int s = g.row_seq ? g.row_seq[t] : t;
+    const bool seq_ok = s >= 0 && s < g.n_seq;
+    r0[r] = !seq_ok ? t : (g.seq_rows ? g.seq_rows[s] : t);
+    const int slot = seq_ok ? g.slots[s] : -1;
+    live[r] = t0 + r < g.T && slot >= 0 && slot < g.n_slots && r0[r] >= 0 && r0[r] <= t;
+    p[r] = g.pos[t];
+    p0[r] = p[r] - (t - r0[r]);
+    tail[r] = (const T*)g.tail + (int64_t)(live[r] ? slot : 0) * m * C;
+    kvs[r] = live[r] ? g.kv_slots[t] : -1;
+  }
+  extern __shared__ float cs_sn[];  // per row [half] cosines, [half] sines of its angles
+  for (int i = threadIdx.x; i < kConvRows * g.half; i += blockDim.x) {
+    const int r = i / g.half, e = i - r * g.half;
+    sincosf((float)p[r] * g.inv_freq[e], &cs_sn[(2 * r + 1) * g.half + e], &cs_sn[2 * r * g.half + e]);
+  }
+  __syncthreads();
+  const int qk = (g.n_q + g.n_k) * g.d, nq = g.n_q * g.d;
+  auto put = [&](int r, int c, const float* y) {
+    if (t0 + r >= g.T) return;
+    if (c < nq) VecIO<T, V>::st((T*)g.q_out + (int64_t)(t0 + r) * nq + c, y);
+    else if (kvs[r] < 0) return;
+    else if (c < qk) VecIO<T, V>::st((T*)g.kc + kvs[r] * (g.n_k * g.d) + (c - nq), y);
+    else VecIO<T, V>::st((T*)g.vc + kvs[r] * (g.n_k * g.dv) + (c - qk), y);
+  };
+  // work items: per q / k head its rotated pairs of runs (a run of the low half with its partner of
+  // the high half), then its runs that are not rotated; then the runs of v
+  const int n_pair = g.half / V, per_head = n_pair + (g.d - 2 * g.half) / V;
+  const int n_head_items = (g.n_q + g.n_k) * per_head, n_items = n_head_items + (C - qk) / V;
+  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+    int c, e;
+    bool pair = false;
+    if (it < n_head_items) {
+      const int hd = it / per_head, j = it - hd * per_head;
+      pair = j < n_pair;
+      e = pair ? j * V : 2 * g.half + (j - n_pair) * V;
+      c = hd * g.d + e;
+    } else {
+      e = 0;
+      c = qk + (it - n_head_items) * V;
+    }
+    float y[kConvRows][V], z[kConvRows][V];
+#pragma unroll
+    for (int r = 0; r < kConvRows; ++r)
+#pragma unroll
+      for (int i = 0; i < V; ++i) y[r][i] = z[r][i] = 0.f;
     for (int jj = 0; jj < g.taps; ++jj) {
-      const int64_t qp = p - m + jj;
-      if (qp < 0) continue;
-      float u[V], w[V];
-      if (qp >= p0) VecIO<T, V>::ld(x + (int64_t)(r0 + (qp - p0)) * g.xs + c, u);
-      else VecIO<T, V>::ld(tail + (qp - p0 + m) * C + c, u);
+      float w[V], w2[V];
       const float* wp = g.cw + (int64_t)jj * C + c;
 #pragma unroll
       for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4*>(w + i) = *reinterpret_cast<const f32x4*>(wp + i);
+      if (pair) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) y[i] += w[i] * u[i];
-    }
-  };
-  extern __shared__ float cs_sn[];  // [half] cosines, [half] sines of the row's angles
-  for (int i = threadIdx.x; i < g.half; i += blockDim.x) sincosf((float)p * g.inv_freq[i], &cs_sn[g.half + i], &cs_sn[i]);
-  __syncthreads();
-  const int qk = (g.n_q + g.n_k) * g.d, nq = g.n_q * g.d;
-  const int64_t kvs = live ? g.kv_slots[t] : -1;
-  auto put = [&](int c, const float* y) {
-    if (c < nq) VecIO<T, V>::st((T*)g.q_out + (int64_t)t * nq + c, y);
-    else if (kvs < 0) return;
-    else if (c < qk) VecIO<T, V>::st((T*)g.kc + kvs * (g.n_k * g.d) + (c - nq), y);
-    else VecIO<T, V>::st((T*)g.vc + kvs * (g.n_k * g.dv) + (c - qk), y);
-  };
-  for (int c = threadIdx.x * V; c < C; c += blockDim.x * V) {
-    const int e = c < qk ? c % g.d : 2 * g.half;
-    if (e >= g.half && e < 2 * g.half) continue;  // the high half rides with its low partner
-    float y[V];
-    conv(c, y);
-    if (e < g.half) {
-      float z[V], lo[V], hi[V];
-      conv(c + g.half, z);
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        const float cs = cs_sn[e + i], sn = cs_sn[g.half + e + i];
-        lo[i] = y[i] * cs - z[i] * sn;
-        hi[i] = z[i] * cs + y[i] * sn;
+        for (int i = 0; i < V; i += 4)
+          *reinterpret_cast<f32x4*>(w2 + i) = *reinterpret_cast<const f32x4*>(wp + g.half + i);
       }
-      put(c, lo);
-      put(c + g.half, hi);
-    } else {
-      put(c, y);
+#pragma unroll
+      for (int r = 0; r < kConvRows; ++r) {
+        const int64_t qp = p[r] - m + jj;
+        if (!live[r] || qp < 0) continue;
+        const T* src = qp >= p0[r] ? x + (int64_t)(r0[r] + (qp - p0[r])) * g.xs + c : tail[r] + (qp - p0[r] + m) * C + c;
+        float u[V];
+        VecIO<T, V>::ld(src, u);
+#pragma unroll
+        for (int i = 0; i < V; ++i) y[r][i] += w[i] * u[i];
+        if (pair) {
+          VecIO<T, V>::ld(src + g.half, u);
+#pragma unroll
+          for (int i = 0; i < V; ++i) z[r][i] += w2[i] * u[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kConvRows; ++r) {
+      if (pair) {
+        float lo[V], hi[V];
+        const float* cs = cs_sn + 2 * r * g.half + e;
+        const float* sn = cs + g.half;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          lo[i] = y[r][i] * cs[i] - z[r][i] * sn[i];
+          hi[i] = z[r][i] * cs[i] + y[r][i] * sn[i];
+        }
+        put(r, c, lo);
+        put(r, c + g.half, hi);
+      } else {
+        put(r, c, y[r]);
+      }
     }
   }
 }
@@ -557,8 +601,9 @@ int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw,
   const bool vec = d % V == 0 && dv % V == 0 && half % V == 0 && xs % V == 0 && al(x) && al(q_out) && al(tail) &&
                    al(kc) && al(vc) && al(cw) && ((n_q * d + n_k * (d + dv)) * esz) % 16 == 0;
   const size_t lds = (size_t)2 * half * sizeof(float);
-  if (vec && f32) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<float, 4>), dim3(T_), dim3(256), lds, st, g);
-  else if (vec) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<bf16_t, 8>), dim3(T_), dim3(256), lds, st, g);
+  const dim3 vgrid((T_ + kConvRows - 1) / kConvRows);
+  if (vec && f32) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<float, 4>), vgrid, dim3(128), kConvRows * lds, st, g);
+  else if (vec) hipLaunchKernelGGL((conv_rope_cache_vec_kernel<bf16_t, 8>), vgrid, dim3(128), kConvRows * lds, st, g);
   else { DISPATCH_T(f32, hipLaunchKernelGGL(conv_rope_cache_kernel<T>, dim3(T_), dim3(256), lds, st, g)); }
   DX_CHECK_LAUNCH();
   return 0;
