@@ -204,52 +204,73 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
     __syncthreads();
     if (t0 + kTok < n) fetch(t0 + kTok);
     const int nt = n - t0 < kTok ? n - t0 : kTok;
-    for (int tt = 0; tt < nt; ++tt) {
-      float x[kRows], y[kRows], us[kCols], o_[kCols];
+    // the five row vectors of a token (unit key, decay, removal, key, read-out) and its values
+    auto load = [&](int tt, float (*b)[kRows], float* vj) {
 #pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&su[tt][rq[q / 4]]);
+      for (int q = 0; q < kRows; q += 4) {
+        *reinterpret_cast<f32x4*>(b[0] + q) = *reinterpret_cast<const f32x4*>(&su[tt][rq[q / 4]]);
+        *reinterpret_cast<f32x4*>(b[1] + q) = *reinterpret_cast<const f32x4*>(&sw[tt][rq[q / 4]]);
+        *reinterpret_cast<f32x4*>(b[2] + q) = *reinterpret_cast<const f32x4*>(&sa[tt][rq[q / 4]]);
+        *reinterpret_cast<f32x4*>(b[3] + q) = *reinterpret_cast<const f32x4*>(&sk[tt][rq[q / 4]]);
+        *reinterpret_cast<f32x4*>(b[4] + q) = *reinterpret_cast<const f32x4*>(&sr[tt][rq[q / 4]]);
+      }
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) vj[c] = sv[tt][grp * kCols + c];
+    };
+    auto step = [&](const float (*b)[kRows], const float* vj, float* o_) {
+      float us[kCols];
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
         float a_ = 0.f;
 #pragma unroll
-        for (int q = 0; q < kRows; ++q) a_ += x[q] * S[c][q];
+        for (int q = 0; q < kRows; ++q) a_ += b[0][q] * S[c][q];
         us[c] = group_sum<R>(a_);
       }
-      float vj[kCols];
-#pragma unroll
-      for (int c = 0; c < kCols; ++c) vj[c] = sv[tt][grp * kCols + c];
-#pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sw[tt][rq[q / 4]]);
-#pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sa[tt][rq[q / 4]]);
-#pragma unroll
-      for (int c = 0; c < kCols; ++c)
-#pragma unroll
-        for (int q = 0; q < kRows; ++q) S[c][q] = S[c][q] * x[q] - y[q] * us[c];
-#pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(x + q) = *reinterpret_cast<const f32x4*>(&sk[tt][rq[q / 4]]);
-#pragma unroll
-      for (int q = 0; q < kRows; q += 4) *reinterpret_cast<f32x4*>(y + q) = *reinterpret_cast<const f32x4*>(&sr[tt][rq[q / 4]]);
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
         float a_ = 0.f;
 #pragma unroll
         for (int q = 0; q < kRows; ++q) {
-          S[c][q] += x[q] * vj[c];
-          a_ += y[q] * S[c][q];
+          S[c][q] = S[c][q] * b[1][q] - b[2][q] * us[c] + b[3][q] * vj[c];
+          a_ += b[4][q] * S[c][q];
         }
         o_[c] = group_sum<R>(a_);
       }
-      if (part == 0) {
-        float* op = outp + (int64_t)(t0 + tt) * g.H * g.dv;
-        if constexpr (kCols == 4) {
-          if (out4) *reinterpret_cast<f32x4*>(op) = f32x4{o_[0], o_[1], o_[2], o_[3]};
-        }
-        if (kCols != 4 || !out4) {
+    };
+    auto store = [&](int tt, const float* o_) {
+      float* op = outp + (int64_t)(t0 + tt) * g.H * g.dv;
+      if constexpr (kCols == 4) {
+        if (out4) *reinterpret_cast<f32x4*>(op) = f32x4{o_[0], o_[1], o_[2], o_[3]};
+      }
+      if (kCols != 4 || !out4) {
 #pragma unroll
-          for (int c = 0; c < kCols; ++c)
-            if (j0 + c < g.dv) op[c] = o_[c];
-        }
+        for (int c = 0; c < kCols; ++c)
+          if (j0 + c < g.dv) op[c] = o_[c];
+      }
+    };
+    if (kCols == 2 && nt == kTok) {
+      // a whole block of the narrow tile (the wide one has no registers to spare), unrolled in one basic
+      // block: the next token's vectors are read from LDS while the current token's chain runs, and the
+      // outputs are stored once at the end
+      float b0[5][kRows], b1[5][kRows], v0[kCols], v1[kCols], ob[kTok][kCols];
+      load(0, b0, v0);
+#pragma unroll
+      for (int tt = 0; tt < kTok; tt += 2) {
+        load(tt + 1, b1, v1);
+        step(b0, v0, ob[tt]);
+        if (tt + 2 < kTok) load(tt + 2, b0, v0);
+        step(b1, v1, ob[tt + 1]);
+      }
+      if (part == 0) {
+#pragma unroll
+        for (int tt = 0; tt < kTok; ++tt) store(tt, ob[tt]);
+      }
+    } else {
+      for (int tt = 0; tt < nt; ++tt) {
+        float b0[5][kRows], v0[kCols], o_[kCols];
+        load(tt, b0, v0);
+        step(b0, v0, o_);
+        if (part == 0) store(tt, o_);
       }
     }
   }
@@ -275,9 +296,13 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
 template <typename T, int R, int CT>
 void launch_delta_ct(const DeltaArgs& g, int n_seq, hipStream_t st) {
   const int need = R * ((g.dv + CT - 1) / CT);
-  if (need <= 64) {
-    hipLaunchKernelGGL((delta_rule_kernel<T, R, 64, CT>), dim3(n_seq, g.H, 1), dim3(64), 0, st, g);
-  } else {
+  if constexpr (R < 16) {  // (a single wave staging 256 key channels would spill its registers)
+    if (need <= 64) {
+      hipLaunchKernelGGL((delta_rule_kernel<T, R, 64, CT>), dim3(n_seq, g.H, 1), dim3(64), 0, st, g);
+      return;
+    }
+  }
+  {
     const int cols = 256 / R * CT;
     hipLaunchKernelGGL((delta_rule_kernel<T, R, 256, CT>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(256), 0,
                        st, g);
