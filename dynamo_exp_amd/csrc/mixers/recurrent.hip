@@ -35,8 +35,9 @@ __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-
 // neighbouring lanes share the columns and join their partial dot products by
 // DPP lane exchanges (no LDS traffic), and a workgroup of NT threads owns
 // NT / R * CT columns of one (sequence, head).  CT is 4 where the launch has
-// waves to fill the chip and 2 where it has not (a few long prompts): the
-// recurrence is bound by instruction issue, so it wants every SIMD busy.  The
+// waves to fill the chip twice over, else 2 or 1 (a few long prompts): a
+// token's dependent chain leaves a lone wave on a SIMD waiting most of the
+// time, so the launch wants at least two waves on every SIMD.  The
 // state tensor is stored column-major per head ([slots, H, dv, dk]) so that a
 // wave's state traffic is contiguous runs.  What the recurrence needs per
 // token and key channel beside r and k -- the unit key u, the decay w and
@@ -248,7 +249,7 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
           if (j0 + c < g.dv) op[c] = o_[c];
       }
     };
-    if (kCols == 2 && nt == kTok) {
+    if (kCols <= 2 && nt == kTok) {
       // a whole block of the narrow tile (the wide one has no registers to spare), unrolled in one basic
       // block: the next token's vectors are read from LDS while the current token's chain runs, and the
       // outputs are stored once at the end
@@ -291,8 +292,9 @@ __global__ void __launch_bounds__(NT) delta_rule_kernel(DeltaArgs g) {
   }
 }
 
-// NT threads per workgroup: 64 where that covers all columns of a head, else 256.  CT = 2 when
-// tiles of four columns would leave the launch under one wave per SIMD (1024 on the chip).
+// NT threads per workgroup: 64 where that covers all columns of a head, else 256.  Columns per
+// thread: the widest tile that still gives the launch two waves per SIMD (2048 on the chip) -- a
+// token's chain leaves a lone wave waiting most of the time -- down to one column for a few long prompts.
 template <typename T, int R, int CT>
 void launch_delta_ct(const DeltaArgs& g, int n_seq, hipStream_t st) {
   const int need = R * ((g.dv + CT - 1) / CT);
@@ -311,8 +313,9 @@ void launch_delta_ct(const DeltaArgs& g, int n_seq, hipStream_t st) {
 template <typename T, int R>
 void launch_delta(const DeltaArgs& g, int n_seq, hipStream_t st) {
   const int64_t waves4 = (int64_t)n_seq * g.H * ((R * ((g.dv + 3) / 4) + 63) / 64);
-  if (waves4 >= 1024) launch_delta_ct<T, R, 4>(g, n_seq, st);
-  else launch_delta_ct<T, R, 2>(g, n_seq, st);
+  if (waves4 >= 2048) launch_delta_ct<T, R, 4>(g, n_seq, st);
+  else if (waves4 >= 1024) launch_delta_ct<T, R, 2>(g, n_seq, st);
+  else launch_delta_ct<T, R, 1>(g, n_seq, st);
 }
 
 // ---------------------------------------------------------------------------
