@@ -558,23 +558,67 @@ __global__ void __launch_bounds__(256) conv_state_update_kernel(T* __restrict__ 
   }
 }
 
-// out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate): one wave per (row, head)
-template <typename T>
-__global__ void __launch_bounds__(64) head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
-                                                            const float* __restrict__ w, const T* __restrict__ gate,
-                                                            int64_t gs, int H, int dv, float eps) {
-  const int64_t v = blockIdx.x;
+// out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate): one wave per (row, head), four per workgroup;
+// a lane keeps its elements (V neighbours at a time, up to kHnKeep times) in registers between the mean
+// square and the result.  V = 2 needs an even dv and gate stride and 8-byte aligned o and w.
+constexpr int kHnKeep = 4;
+template <typename T, int V>
+__global__ void __launch_bounds__(256) head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                                             const float* __restrict__ w, const T* __restrict__ gate,
+                                                             int64_t gs, int64_t n_vec, int H, int dv, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (v >= n_vec) return;
   const int64_t row = v / H;
   const int h = (int)(v - row * H);
   const float* op = o + v * dv;
-  float ss = 0.f;
-  for (int e = threadIdx.x; e < dv; e += 64) ss += op[e] * op[e];
+  auto ldo = [&](int e, float* x) {
+    if constexpr (V == 2) {
+      const float2 t = *reinterpret_cast<const float2*>(op + e);
+      x[0] = t.x, x[1] = t.y;
+    } else {
+      x[0] = op[e];
+    }
+  };
+  float x[kHnKeep][V], ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kHnKeep; ++k) {
+    const int e = (lane + 64 * k) * V;
+#pragma unroll
+    for (int i = 0; i < V; ++i) x[k][i] = 0.f;
+    if (e < dv) ldo(e, x[k]);
+#pragma unroll
+    for (int i = 0; i < V; ++i) ss += x[k][i] * x[k][i];
+  }
+  for (int e = (lane + 64 * kHnKeep) * V; e < dv; e += 64 * V) {
+    float t[V];
+    ldo(e, t);
+#pragma unroll
+    for (int i = 0; i < V; ++i) ss += t[i] * t[i];
+  }
   const float inv = rsqrtf(wave_reduce_sum(ss) / (float)dv + eps);
-  for (int e = threadIdx.x; e < dv; e += 64) {
-    float y = op[e] * inv;
-    if (w) y *= w[h * dv + e];
-    if (gate) y *= sigmoidf_(ldf<T>(gate, row * gs + h * dv + e));
-    stf<T>(out, v * dv + e, y);
+  auto put = [&](int e, const float* xv) {
+    float y[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      y[i] = xv[i] * inv;
+      if (w) y[i] *= w[h * dv + e + i];
+      if (gate) y[i] *= sigmoidf_(ldf<T>(gate, row * gs + h * dv + e + i));
+    }
+    if constexpr (V == 2 && sizeof(T) == 2) {
+      *reinterpret_cast<uint32_t*>((bf16_t*)out + v * dv + e) = pack_bf16x2(y[0], y[1]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < V; ++i) stf<T>(out, v * dv + e + i, y[i]);
+    }
+  };
+#pragma unroll
+  for (int k = 0; k < kHnKeep; ++k)
+    if ((lane + 64 * k) * V < dv) put((lane + 64 * k) * V, x[k]);
+  for (int e = (lane + 64 * kHnKeep) * V; e < dv; e += 64 * V) {
+    float t[V];
+    ldo(e, t);
+    put(e, t);
   }
 }
 
@@ -652,8 +696,16 @@ int dxm_head_norm_gate(void* out, const float* o, const float* w, const void* ga
                        int dv, float eps, int f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (H < 1 || dv < 1 || (int64_t)rows * H > 0x7fffffff) return 1;
-  DISPATCH_T(f32, hipLaunchKernelGGL(head_norm_gate_kernel<T>, dim3((unsigned)(rows * H)), dim3(64), 0, st, (T*)out, o,
-                                     w, (const T*)gate, gs, H, dv, eps));
+  const int64_t n_vec = (int64_t)rows * H;
+  const dim3 grid((unsigned)((n_vec + 3) / 4));
+  const bool v2 = dv % 2 == 0 && gs % 2 == 0 && (uintptr_t)o % 8 == 0 && (uintptr_t)out % 4 == 0;
+  if (v2) {
+    DISPATCH_T(f32, hipLaunchKernelGGL((head_norm_gate_kernel<T, 2>), grid, dim3(256), 0, st, (T*)out, o, w,
+                                       (const T*)gate, gs, n_vec, H, dv, eps));
+  } else {
+    DISPATCH_T(f32, hipLaunchKernelGGL((head_norm_gate_kernel<T, 1>), grid, dim3(256), 0, st, (T*)out, o, w,
+                                       (const T*)gate, gs, n_vec, H, dv, eps));
+  }
   DX_CHECK_LAUNCH();
   return 0;
 }
