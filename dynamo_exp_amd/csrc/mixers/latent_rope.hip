@@ -1,0 +1,108 @@
+// Query / key preparation of latent attention with a rotated key part, for
+// gfx950: per token row
+//   * the latent (the first r columns of the down-projection) is RMS-normed with
+//     a weight per column and written to the paged cache row [0, r);
+//   * the key part that carries the position (the next dr columns, not normed,
+//     shared by all heads) is rotated and written to the cache row [r, r + dr);
+//   * every head's query is assembled as [qa_h (r) | rotate(q_h's last dr columns)]:
+//     qa is the head's unrotated query part already multiplied by the head's key
+//     up-projection, so that q' . [latent | rotated key] is the head's score.
+// The cache row [latent | rotated key] is key and (its first r columns) value
+// of one shared head.
+//
+// Rotation: the first 2 * half columns of a dr-wide part, column i paired with
+// i + half, angle = position * inv_freq[i] (fp32, sincosf), cosine and sine
+// both multiplied by `mag`; columns from 2 * half on pass unchanged.
+// Norm sums, angles and the rotation are fp32 whatever the element type is.
+#include "../kernels/common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+
+struct LatentArgs {
+  void* q_out;      // [T, H, r + dr]
+  const void* qa;   // [H, T, r]: unrotated query parts times the key up-projection
+  const void* q;    // [T, q_stride]: head h's rotated part at columns h * q_head + q_off .. + dr
+  int64_t q_stride;
+  int q_head, q_off;
+  const void* kv;   // [T, kv_stride]: [latent (r) | rotated key part (dr)]
+  int64_t kv_stride;
+  const float* cn;  // [r] latent norm weight
+  float eps;
+  const float* inv_freq;  // [half]
+  int half;
+  float mag;
+  const int64_t* pos;
+  const int64_t* slots;  // cache row of every token (-1: not cached)
+  void* cache;           // [slots, r + dr]
+  int T, H, r, dr;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) latent_rope_kernel(LatentArgs g) {
+  extern __shared__ float cs_sn[];  // [half] cosines, [half] sines, both times mag
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float p = (float)g.pos[t];
+  for (int i = tid; i < g.half; i += blockDim.x) {
+    float sn, cs;
+    sincosf(p * g.inv_freq[i], &sn, &cs);
+    cs_sn[i] = cs * g.mag;
+    cs_sn[g.half + i] = sn * g.mag;
+  }
+  const T* kv = (const T*)g.kv + t * g.kv_stride;
+  float ss = 0.f;
+  for (int c = tid; c < g.r; c += blockDim.x) {
+    const float x = ldf<T>(kv, c);
+    ss += x * x;
+  }
+  const float rs = rsqrtf(block_reduce_sum(ss, red) / (float)g.r + g.eps);  // (also orders the LDS writes above)
+  const int Wc = g.r + g.dr;
+  // rotated value of column e (< dr) of a dr-wide part at src
+  auto rot = [&](const T* src, int e) -> float {
+    const float x = ldf<T>(src, e);
+    if (e >= 2 * g.half) return x;
+    const int i = e < g.half ? e : e - g.half;
+    const float other = ldf<T>(src, e < g.half ? e + g.half : e - g.half);
+    return e < g.half ? x * cs_sn[i] - other * cs_sn[g.half + i] : x * cs_sn[i] + other * cs_sn[g.half + i];
+  };
+  const int64_t slot = g.slots[t];
+  if (slot >= 0) {
+    T* row = (T*)g.cache + slot * Wc;
+    for (int c = tid; c < g.r; c += blockDim.x) stf<T>(row, c, ldf<T>(kv, c) * rs * g.cn[c]);
+    for (int e = tid; e < g.dr; e += blockDim.x) stf<T>(row, g.r + e, rot(kv + g.r, e));
+  }
+  const T* q = (const T*)g.q + t * g.q_stride;
+  T* qo = (T*)g.q_out + t * (int64_t)g.H * Wc;
+  for (int it = tid; it < g.H * Wc; it += blockDim.x) {
+    const int h = it / Wc, c = it - h * Wc;
+    if (c < g.r) qo[it] = ((const T*)g.qa)[((int64_t)h * g.T + t) * g.r + c];
+    else stf<T>(qo, it, rot(q + (int64_t)h * g.q_head + g.q_off, c - g.r));
+  }
+}
+
+}  // namespace
+
+extern "C" int dxm_latent_rope(void* q_out, const void* qa, const void* q, int64_t q_stride, int q_head, int q_off,
+                               const void* kv, int64_t kv_stride, const float* cn, float eps, const float* inv_freq,
+                               int half, float mag, const int64_t* pos, const int64_t* slots, void* cache, int T_, int H,
+                               int r, int dr, int f32, hipStream_t st) {
+  if (T_ <= 0) return 0;
+  if (H < 1 || r < 1 || dr < 0 || half < 0 || 2 * half > dr || half > 4096) return 1;
+  if (!q_out || !qa || !kv || !cn || !pos || !slots || !cache || (dr && !q) || (half && !inv_freq)) return 2;
+  if (q_off < 0 || q_off + dr > q_head) return 3;
+  LatentArgs g{q_out, qa, q, q_stride, q_head, q_off, kv, kv_stride, cn, eps, inv_freq, half, mag,
+               pos, slots, cache, T_, H, r, dr};
+  const size_t lds = (size_t)2 * half * sizeof(float);
+  if (f32) hipLaunchKernelGGL(latent_rope_kernel<float>, dim3(T_), dim3(256), lds, st, g);
+  else hipLaunchKernelGGL(latent_rope_kernel<bf16_t>, dim3(T_), dim3(256), lds, st, g);
+  DX_CHECK_LAUNCH();
+  return 0;
+}

@@ -1,5 +1,5 @@
 // Kernels with per-sequence state for gfx950: the generalized delta rule (a
-// running matrix per head), short causal convolutions over time fused with
+// running matrix per head), retention (a fixed decay per head), short causal convolutions over time fused with
 // rotary positions and the paged cache write, the convolution tail update, and
 // the per-head unit-RMS + gate that follows a recurrent mixer.
 //
@@ -319,6 +319,109 @@ void launch_delta(const DeltaArgs& g, int n_seq, hipStream_t st) {
 }
 
 // ---------------------------------------------------------------------------
+// Retention: linear attention with one fixed decay per head, no softmax and no
+// denominator.  Per (sequence, head) a matrix S [dk, dv]:
+//     S_t = decay_h S_(t-1) + (k_scale k_t) v_t^T,   o_t = S_t^T q_t.
+// Columns of S are independent: R neighbouring lanes share a column (lane r of
+// the group owns rows r, r + R, ..., up to kRows of them, in registers) and join
+// their partial q^T S by DPP lane exchanges; a workgroup owns blockDim / R
+// columns of one (sequence, head).  Tokens are staged through LDS kTok at a
+// time (q, scaled k: [kTok][dk]; v: [kTok][columns]).  State layout as for the
+// delta rule: [slots, H, dv, dk], a column's rows contiguous.
+struct RetArgs {
+  float* out;    // [T, H * dv]
+  float* state;  // [slots, H, dv, dk]
+  const void *q, *k, *v;
+  int64_t qs, ks, vs;  // row strides (elements)
+  const float* decay;  // [H]
+  float k_scale;
+  const int64_t* pos;
+  const int* seq_rows;  // null: row i is sequence i
+  const int* slots;
+  int n_slots, T, H, dk, dv;
+};
+
+template <typename T, int R>
+__global__ void __launch_bounds__(256) retention_kernel(RetArgs g) {
+  extern __shared__ float ret_lds[];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, cols = blockDim.x / R;
+  const int cl = tid / R, r = tid % R;
+  const int col0 = blockIdx.z * cols, j = col0 + cl;
+  const int r0 = g.seq_rows ? g.seq_rows[s] : s, r1 = g.seq_rows ? g.seq_rows[s + 1] : s + 1;
+  if (r1 <= r0 || r0 < 0 || r1 > g.T) return;
+  const bool colok = j < g.dv;
+  const int slot = g.slots[s];
+  const int64_t ow = (int64_t)g.H * g.dv;
+  if (slot < 0 || slot >= g.n_slots) {  // a padding row: zeros out, no state touched
+    for (int t = r0; t < r1; ++t)
+      if (r == 0 && colok) g.out[(int64_t)t * ow + h * g.dv + j] = 0.f;
+    return;
+  }
+  float* qs_ = ret_lds;
+  float* ks_ = qs_ + kTok * g.dk;
+  float* vs_ = ks_ + kTok * g.dk;
+  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv + (colok ? j : 0)) * g.dk;
+  const bool fresh = g.pos[r0] == 0;
+  float S[kRows];
+#pragma unroll
+  for (int ii = 0; ii < kRows; ++ii) {
+    const int i = r + R * ii;
+    S[ii] = (!fresh && colok && i < g.dk) ? sp[i] : 0.f;
+  }
+  const float dec = g.decay[h];
+  const T* q = (const T*)g.q;
+  const T* k = (const T*)g.k;
+  const T* v = (const T*)g.v;
+  for (int t0 = r0; t0 < r1; t0 += kTok) {
+    const int nt = r1 - t0 < kTok ? r1 - t0 : kTok;
+    __syncthreads();  // the previous block's reads are done
+    for (int e = tid; e < nt * g.dk; e += blockDim.x) {
+      const int tt = e / g.dk, i = e - tt * g.dk;
+      qs_[e] = ldf<T>(q, (int64_t)(t0 + tt) * g.qs + h * g.dk + i);
+      ks_[e] = ldf<T>(k, (int64_t)(t0 + tt) * g.ks + h * g.dk + i) * g.k_scale;
+    }
+    for (int e = tid; e < nt * cols; e += blockDim.x) {
+      const int tt = e / cols, c = e - tt * cols;
+      vs_[e] = col0 + c < g.dv ? ldf<T>(v, (int64_t)(t0 + tt) * g.vs + h * g.dv + col0 + c) : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vj = vs_[tt * cols + cl];
+      const float* qt = qs_ + tt * g.dk;
+      const float* kt = ks_ + tt * g.dk;
+      float acc = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < kRows; ++ii) {
+        const int i = r + R * ii;
+        if (i < g.dk) {
+          S[ii] = dec * S[ii] + kt[i] * vj;
+          acc += qt[i] * S[ii];
+        }
+      }
+      acc = group_sum<R>(acc);
+      if (r == 0 && colok) g.out[(int64_t)(t0 + tt) * ow + h * g.dv + j] = acc;
+    }
+  }
+  if (colok) {
+#pragma unroll
+    for (int ii = 0; ii < kRows; ++ii) {
+      const int i = r + R * ii;
+      if (i < g.dk) sp[i] = S[ii];
+    }
+  }
+}
+
+template <typename T, int R>
+void launch_retention(const RetArgs& g, int n_seq, hipStream_t st) {
+  int nt = (R * g.dv + 63) / 64 * 64;
+  nt = nt > 256 ? 256 : nt;
+  const int cols = nt / R;
+  const size_t lds = (size_t)(2 * kTok * g.dk + kTok * cols) * sizeof(float);
+  hipLaunchKernelGGL((retention_kernel<T, R>), dim3(n_seq, g.H, (g.dv + cols - 1) / cols), dim3(nt), lds, st, g);
+}
+
+// ---------------------------------------------------------------------------
 // Short causal convolution over time on the leading C = n_q d + n_k (d + dv)
 // columns of a fused projection, then rotary positions on the first 2 * half
 // columns of every q and k head (column i paired with i + half), q to its own
@@ -558,14 +661,15 @@ __global__ void __launch_bounds__(256) conv_state_update_kernel(T* __restrict__ 
   }
 }
 
-// out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate): one wave per (row, head), four per workgroup;
+// out = o / sqrt(mean_head(o^2) + eps) * w * sigmoid(gate) (or * silu(gate)): one wave per (row, head), four per workgroup;
 // a lane keeps its elements (V neighbours at a time, up to kHnKeep times) in registers between the mean
 // square and the result.  V = 2 needs an even dv and gate stride and 8-byte aligned o and w.
 constexpr int kHnKeep = 4;
 template <typename T, int V>
 __global__ void __launch_bounds__(256) head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
                                                              const float* __restrict__ w, const T* __restrict__ gate,
-                                                             int64_t gs, int64_t n_vec, int H, int dv, float eps) {
+                                                             int64_t gs, int64_t n_vec, int H, int dv, float eps,
+                                                             int gate_act) {
   const int lane = threadIdx.x & 63;
   const int64_t v = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (v >= n_vec) return;
@@ -603,7 +707,10 @@ __global__ void __launch_bounds__(256) head_norm_gate_kernel(T* __restrict__ out
     for (int i = 0; i < V; ++i) {
       y[i] = xv[i] * inv;
       if (w) y[i] *= w[h * dv + e + i];
-      if (gate) y[i] *= sigmoidf_(ldf<T>(gate, row * gs + h * dv + e + i));
+      if (gate) {  // gate_act 0: sigmoid(z); 1: silu, z sigmoid(z)
+        const float z = ldf<T>(gate, row * gs + h * dv + e + i);
+        y[i] *= gate_act ? z * sigmoidf_(z) : sigmoidf_(z);
+      }
     }
     if constexpr (V == 2 && sizeof(T) == 2) {
       *reinterpret_cast<uint32_t*>((bf16_t*)out + v * dv + e) = pack_bf16x2(y[0], y[1]);
@@ -657,6 +764,26 @@ int dxm_delta_rule(float* out, float* state, int n_slots, float* prep, const voi
   return 0;
 }
 
+int dxm_retention(float* out, float* state, int n_slots, const void* q, int64_t qs, const void* k, int64_t ks,
+                  const void* v, int64_t vs, const float* decay, float k_scale, const int64_t* pos,
+                  const int* seq_rows, const int* slots, int n_seq, int T_, int H, int dk, int dv, int f32,
+                  hipStream_t st) {
+  if (n_seq <= 0 || T_ <= 0) return 0;
+  if (H < 1 || dk < 1 || dv < 1 || n_slots < 1 || H > 65535 || (int64_t)T_ * H * dv > 0x7fffffffffffLL) return 1;
+  if (dk > kRows * 16) return 2;  // wider keys need more lanes per column than instantiated
+  if (!out || !state || !pos || !slots || !decay || !q || !k || !v) return 3;
+  if (!seq_rows && n_seq != T_) return 4;
+  RetArgs g{out, state, q, k, v, qs, ks, vs, decay, k_scale, pos, seq_rows, slots, n_slots, T_, H, dk, dv};
+  const int need = (dk + kRows - 1) / kRows;
+  if (need <= 1) { DISPATCH_T(f32, (launch_retention<T, 1>(g, n_seq, st))); }
+  else if (need <= 2) { DISPATCH_T(f32, (launch_retention<T, 2>(g, n_seq, st))); }
+  else if (need <= 4) { DISPATCH_T(f32, (launch_retention<T, 4>(g, n_seq, st))); }
+  else if (need <= 8) { DISPATCH_T(f32, (launch_retention<T, 8>(g, n_seq, st))); }
+  else { DISPATCH_T(f32, (launch_retention<T, 16>(g, n_seq, st))); }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
 int dxm_conv_rope_cache(void* q_out, const void* x, int64_t xs, const float* cw, int taps, const void* tail,
                         int n_slots, const int64_t* pos, const int64_t* kv_slots, const int* row_seq,
                         const int* seq_rows, const int* slots, int n_seq, int T_, int n_q, int n_k, int d, int dv,
@@ -693,18 +820,18 @@ int dxm_conv_state_update(void* tail, int n_slots, const void* x, int64_t xs, co
 }
 
 int dxm_head_norm_gate(void* out, const float* o, const float* w, const void* gate, int64_t gs, int rows, int H,
-                       int dv, float eps, int f32, hipStream_t st) {
+                       int dv, float eps, int gate_act, int f32, hipStream_t st) {
   if (rows <= 0) return 0;
-  if (H < 1 || dv < 1 || (int64_t)rows * H > 0x7fffffff) return 1;
+  if (H < 1 || dv < 1 || (int64_t)rows * H > 0x7fffffff || gate_act < 0 || gate_act > 1) return 1;
   const int64_t n_vec = (int64_t)rows * H;
   const dim3 grid((unsigned)((n_vec + 3) / 4));
   const bool v2 = dv % 2 == 0 && gs % 2 == 0 && (uintptr_t)o % 8 == 0 && (uintptr_t)out % 4 == 0;
   if (v2) {
     DISPATCH_T(f32, hipLaunchKernelGGL((head_norm_gate_kernel<T, 2>), grid, dim3(256), 0, st, (T*)out, o, w,
-                                       (const T*)gate, gs, n_vec, H, dv, eps));
+                                       (const T*)gate, gs, n_vec, H, dv, eps, gate_act));
   } else {
     DISPATCH_T(f32, hipLaunchKernelGGL((head_norm_gate_kernel<T, 1>), grid, dim3(256), 0, st, (T*)out, o, w,
-                                       (const T*)gate, gs, n_vec, H, dv, eps));
+                                       (const T*)gate, gs, n_vec, H, dv, eps, gate_act));
   }
   DX_CHECK_LAUNCH();
   return 0;

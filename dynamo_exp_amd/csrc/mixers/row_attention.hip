@@ -6,6 +6,8 @@
 // sequences side by side, and the visible keys of a row at position p are
 //     causal:  0 .. p          window: max(0, p - size + 1) .. p
 //     chunk:   floor(p / size) * size .. p
+// and, for a window with `keep` > 0, also the sequence's first `keep` keys
+// (0 .. keep - 1, at their true positions) however far back they lie,
 // counted in sequence positions, so the result does not depend on how a prompt
 // was cut into steps.  The score of query position p and key position j is
 // s = q . k * scale, optionally capped, s <- cap * tanh(s / cap), and optionally
@@ -19,6 +21,9 @@
 // (qh / maps / group) * maps + qh % maps and V head qh / maps / group
 // (group = query heads per key/value head): maps = 1 is grouped-query
 // attention, maps = 2 the two score maps of differential attention.
+//
+// With `sink` (a number per query vector) a softmax's denominator also holds
+// exp(sink): a key without a value that is neither scaled nor masked, counted once.
 //
 // Work split: 64 keys per tile, one key per lane for the scores (the query
 // sits in LDS as fp32, pre-scaled), then the lanes turn to the value columns
@@ -77,6 +82,8 @@ struct RowAttnArgs {
   const float* hbias;   // [n_qh] added to the score (null: none)
   const void* gate;     // [rows, gate_stride] logits per head: the result is multiplied by sigmoid (null: none)
   int64_t gate_stride;
+  int keep;           // window mask: the first `keep` keys of the sequence stay visible (0: none)
+  const float* sink;  // [n_qh] softmax only: exp(sink) joins the denominator (null: none)
 };
 
 template <typename T, typename OutT, int NV>
@@ -97,7 +104,9 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
   __syncthreads();
   const T* kc = (const T*)a.kc + (int64_t)kh * a.d;
   const T* vc = (const T*)a.vc + (int64_t)g * a.dv;
-  const int64_t n_keys = p - lo + 1;
+  // visible keys in one numbering u = 0 .. n_keys - 1: the kept first nf keys, then lo .. p
+  const int64_t nf = a.mask == 1 && a.keep > 0 ? (a.keep < lo ? a.keep : lo) : 0;
+  const int64_t n_keys = nf + p - lo + 1;
   const int64_t tiles = (n_keys + 63) / 64;
   const int64_t tpp = (tiles + a.parts - 1) / a.parts;
   const int64_t t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
@@ -110,8 +119,9 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
 #pragma unroll
   for (int c = 0; c < NV; ++c) acc[c] = 0.f;
   for (int64_t t = t0; t < t1; ++t) {
-    const int64_t j = lo + t * 64 + lane;
-    const bool ok = j <= p;
+    const int64_t u = t * 64 + lane;
+    const int64_t j = u < nf ? u : lo + (u - nf);
+    const bool ok = u < n_keys;
     int slot = 0;
     float s = -INFINITY;
     if (ok) {
@@ -139,7 +149,7 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
 #pragma unroll
       for (int c = 0; c < NV; ++c) acc[c] *= alpha;
     }
-    const int64_t left = p - (lo + t * 64) + 1;
+    const int64_t left = n_keys - t * 64;
     const int n = left < 64 ? (int)left : 64;
     for (int jj = 0; jj < n; ++jj) {
       const float wj = __shfl(w, jj, 64);
@@ -154,6 +164,7 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
   }
   if (a.parts == 1) {
     OutT* o = (OutT*)a.out + ((int64_t)row * a.n_qh + qh) * a.dv;
+    if (a.sink && !a.wfn) l += expf(a.sink[qh] - mx);
     float inv = 1.f / l;
     if (a.gate) inv /= 1.f + expf(-Elem<T>::ld((const T*)a.gate, (int64_t)row * a.gate_stride + head));
 #pragma unroll
@@ -178,11 +189,12 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
 // joins the per-part (max, sum, acc) of one (row, head): one wave each
 // (sigmoid weights: every part carries max 0 and sum 1, so the join is the plain sum of the
 // parts divided by their number -- `plain` undoes that division); gate: logits [rows, gs] per
-// head, the result is multiplied by their sigmoid
+// head, the result is multiplied by their sigmoid; sink: [n_qh], exp(sink) joins the softmax denominator once
 template <typename OutT, typename GT>
 __global__ void __launch_bounds__(64) merge_parts_kernel(OutT* __restrict__ out, const float* __restrict__ ws,
                                                          int parts, int dv, int plain, const GT* __restrict__ gate,
-                                                         int64_t gs, int n_qh, int maps) {
+                                                         int64_t gs, int n_qh, int maps,
+                                                         const float* __restrict__ sink) {
   const int lane = threadIdx.x;
   const int64_t v = blockIdx.x;
   const float* w = ws + v * parts * (int64_t)(2 + dv);
@@ -199,6 +211,7 @@ __global__ void __launch_bounds__(64) merge_parts_kernel(OutT* __restrict__ out,
     const float* wp = w + (int64_t)p * (2 + dv);
     if (wp[1] > 0.f) l += wp[1] * __expf(wp[0] - mx);
   }
+  if (sink && !plain) l += expf(sink[v % n_qh] - mx);
   const float inv = post / l;
   for (int e = lane; e < dv; e += 64) {
     float acc = 0.f;
@@ -232,7 +245,7 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
     else hipLaunchKernelGGL((row_attention_kernel<T, OutT, 16>), grid, dim3(64), lds, st, b);
     if (a.parts > 1)
       hipLaunchKernelGGL((merge_parts_kernel<OutT, T>), dim3((unsigned)nr * a.n_qh), dim3(64), 0, st, (OutT*)b.out, b.ws,
-                         a.parts, a.dv, a.wfn, (const T*)b.gate, a.gate_stride, a.n_qh, a.maps);
+                         a.parts, a.dv, a.wfn, (const T*)b.gate, a.gate_stride, a.n_qh, a.maps, a.sink);
   }
   DX_CHECK_LAUNCH();
   return 0;
@@ -244,16 +257,16 @@ extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_
                                  const int64_t* pos, const int* seq, const int* bt, int bt_stride, int bs, int rows,
                                  int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
                                  int size, float softcap, const float* r1, const float* r2, int wfn, const float* hbias,
-                                 const void* gate, int64_t gate_stride, int parts, int f32, int out_f32,
-                                 hipStream_t st) {
+                                 const void* gate, int64_t gate_stride, int keep, const float* sink, int parts, int f32,
+                                 int out_f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group) return 1;
   if (d < 1 || dv < 1 || dv > 1024 || d > 8192) return 2;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535 || n_qh > 65535) return 3;
   if (parts > 1 && !ws) return 4;
-  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1 || keep < 0 || (keep && mask != 1)) return 6;
   RowAttnArgs a{q, q_stride, kc, vc, out, ws, pos, seq, bt, bt_stride, bs, n_qh, maps, group,
-                d, dv, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias, gate, gate_stride};
+                d, dv, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias, gate, gate_stride, keep, sink};
   if (f32) return launch_rows<float, float>(a, rows, st);
   if (out_f32) return launch_rows<bf16_t, float>(a, rows, st);
   return launch_rows<bf16_t, bf16_t>(a, rows, st);
@@ -262,16 +275,16 @@ extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_
 // out [n_vec, dv] (bf16 or fp32) from per-part partials ws [n_vec, parts, 2 + dv]; n_vec = rows * n_qh;
 // plain: the parts hold sigmoid-weighted sums (max 0, sum 1 each); gate: bf16 logits [rows, gate_stride]
 extern "C" int dxm_merge_parts(void* out, const float* ws, int64_t n_vec, int parts, int dv, int plain,
-                               const void* gate, int64_t gate_stride, int n_qh, int maps, int out_f32,
-                               hipStream_t st) {
+                               const void* gate, int64_t gate_stride, int n_qh, int maps, const float* sink,
+                               int out_f32, hipStream_t st) {
   if (n_vec <= 0) return 0;
   if (parts < 1 || dv < 1 || n_vec > 0x7fffffff || n_qh < 1 || maps < 1) return 1;
   if (out_f32)
     hipLaunchKernelGGL((merge_parts_kernel<float, bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (float*)out, ws,
-                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps);
+                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps, sink);
   else
     hipLaunchKernelGGL((merge_parts_kernel<bf16_t, bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (bf16_t*)out, ws,
-                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps);
+                       parts, dv, plain, (const bf16_t*)gate, gate_stride, n_qh, maps, sink);
   DX_CHECK_LAUNCH();
   return 0;
 }

@@ -146,20 +146,21 @@ __global__ void __launch_bounds__(kThreads) stream_step_kernel(float* __restrict
   }
 }
 
-// X[t, s, :] = table[ids[t], :] (+ ptab[pos[t], :], a learned vector per position)
-// for every stream s (fp32 streams; the sum is fp32)
+// X[t, s, :] = table[ids[t], :] * scale (+ ptab[pos[t], :], a learned vector per position)
+// for every stream s (fp32 streams; product and sum are fp32)
 template <typename T>
 __global__ void __launch_bounds__(kThreads) embed_streams_kernel(float* __restrict__ X, const T* __restrict__ table,
                                                                  const int64_t* __restrict__ ids, int S, int W,
                                                                  int64_t vocab, const T* __restrict__ ptab,
-                                                                 const int64_t* __restrict__ pos, int64_t n_pos) {
+                                                                 const int64_t* __restrict__ pos, int64_t n_pos,
+                                                                 float scale) {
   const int64_t t = blockIdx.x;
   const int64_t id = ids[t];
   const bool ok = id >= 0 && id < vocab;
   const int64_t p = ptab ? pos[t] : -1;
   const bool pok = p >= 0 && p < n_pos;
   for (int c = threadIdx.x; c < W; c += kThreads) {
-    float v = ok ? ldf<T>(table, id * (int64_t)W + c) : 0.f;
+    float v = ok ? ldf<T>(table, id * (int64_t)W + c) * scale : 0.f;
     if (pok) v += ldf<T>(ptab, p * (int64_t)W + c);
     for (int s = 0; s < S; ++s) X[(t * S + s) * (int64_t)W + c] = v;
   }
@@ -334,6 +335,99 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
   }
 }
 
+// Weighted sum over the results of all layers so far (a depth average):
+//     dst[r, :] = sum_{j < n} w[j] * stack[j][row(r), :]        row(r) = rows ? rows[r] : r
+// stack [>= n, T, W] fp32, one [T, W] plane per layer result; dst fp32 [n_rows, W] (it may be a
+// later plane of the same stack); then, when out: out = dst / sqrt(mean(dst^2) + eps) * nw in T
+// (nw one weight per column).  Sums in the order j = 0, 1, ..., all fp32.  The row stays in
+// registers between the sum and the norm (W <= kThreads * V * kResChunks) or is re-read from dst.
+template <typename T, int V>
+__global__ void __launch_bounds__(kThreads) depth_mix_kernel(float* __restrict__ dst, const float* __restrict__ stack,
+                                                             int64_t plane, int n, const float* __restrict__ w,
+                                                             const int64_t* __restrict__ rows, float eps,
+                                                             const float* __restrict__ nw, T* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t row = rows ? rows[r] : r;
+  const float* src = stack + row * (int64_t)W;
+  float* x = dst + r * (int64_t)W;
+  float acc[kResChunks][V];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kResChunks; ++k) {
+    const int e = (threadIdx.x + k * kThreads) * V;
+    if (e < W) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[k][i] = 0.f;
+      for (int j = 0; j < n; ++j) {
+        float t[V];
+        ldv<float, V>(src + j * plane + e, t);
+        const float wj = w[j];
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[k][i] += wj * t[i];
+      }
+      stv<float, V>(x + e, acc[k]);
+#pragma unroll
+      for (int i = 0; i < V; ++i) ss += acc[k][i] * acc[k][i];
+    }
+  }
+  for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
+    float a[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) a[i] = 0.f;
+    for (int j = 0; j < n; ++j) {
+      float t[V];
+      ldv<float, V>(src + j * plane + e, t);
+      const float wj = w[j];
+#pragma unroll
+      for (int i = 0; i < V; ++i) a[i] += wj * t[i];
+    }
+    stv<float, V>(x + e, a);
+#pragma unroll
+    for (int i = 0; i < V; ++i) ss += a[i] * a[i];
+  }
+  if (!out) return;
+  const float rs = rsqrtf(block_reduce_sum(ss, red) / (float)W + eps);
+#pragma unroll
+  for (int k = 0; k < kResChunks; ++k) {
+    const int e = (threadIdx.x + k * kThreads) * V;
+    if (e < W) {
+      float g[V], o[V];
+      ldv<float, V>(nw + e, g);
+#pragma unroll
+      for (int i = 0; i < V; ++i) o[i] = acc[k][i] * rs * g[i];
+      stv<T, V>(out + r * (int64_t)W + e, o);
+    }
+  }
+  for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
+    float a[V], g[V], o[V];
+    ldv<float, V>(x + e, a);  // written by this thread above
+    ldv<float, V>(nw + e, g);
+#pragma unroll
+    for (int i = 0; i < V; ++i) o[i] = a[i] * rs * g[i];
+    stv<T, V>(out + r * (int64_t)W + e, o);
+  }
+}
+
+// out [rows, n] = x / sqrt(mean(x^2) + eps) * w over a column section x [rows, n] of wider rows
+// (a low-rank latent between its two projections): one wave per row, fp32 sums
+template <typename T>
+__global__ void __launch_bounds__(kThreads) section_norm_kernel(T* __restrict__ out, const T* __restrict__ x,
+                                                                int64_t x_stride, const float* __restrict__ w,
+                                                                int rows, int n, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * x_stride;
+  float ss = 0.f;
+  for (int e = lane; e < n; e += 64) {
+    const float v = ldf<T>(xr, e);
+    ss += v * v;
+  }
+  const float rs = rsqrtf(wave_reduce_sum(ss) / (float)n + eps);
+  for (int e = lane; e < n; e += 64) stf<T>(out, row * n + e, ldf<T>(xr, e) * rs * (w ? w[e] : 1.f));
+}
+
 __device__ __forceinline__ float act_fn(float z, int act) {
   if (act == 5) return tanhf(z);
   if (act == 0) return fmaxf(z, 0.f);           // relu
@@ -454,12 +548,14 @@ __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
 }
 
 // Two-map attention combine: a [rows, H, 2, dv] fp32 (map outputs over the
-// same values)  ->  out [rows, H, dv] = unit_rms(a1 - lam * a2) * post.
+// same values)  ->  out [rows, H, dv] = unit_rms(a1 - lam * a2) * post, times
+// sigmoid(gate[row, head]) when gate (logits [rows, gate_stride], one per head) is given.
 // One wave per (row, head).
 template <typename T>
 __global__ void __launch_bounds__(kThreads) diff_combine_kernel(T* __restrict__ out, const float* __restrict__ a,
                                                                 int64_t n_vec, int dv, float lam, float post,
-                                                                float eps) {
+                                                                float eps, const T* __restrict__ gate,
+                                                                int64_t gate_stride, int H) {
   const int lane = threadIdx.x & 63;
   const int64_t v = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
   if (v >= n_vec) return;
@@ -470,7 +566,8 @@ __global__ void __launch_bounds__(kThreads) diff_combine_kernel(T* __restrict__ 
     const float o = a1[e] - lam * a2[e];
     ss += o * o;
   }
-  const float r = rsqrtf(wave_reduce_sum(ss) / (float)dv + eps) * post;
+  float r = rsqrtf(wave_reduce_sum(ss) / (float)dv + eps) * post;
+  if (gate) r /= 1.f + expf(-ldf<T>(gate, v / H * gate_stride + v % H));
   for (int e = lane; e < dv; e += 64) stf<T>(out, v * dv + e, (a1[e] - lam * a2[e]) * r);
 }
 
@@ -509,11 +606,11 @@ int dxm_stream_step(float* X, const void* y, int64_t y_stride, const float* mix,
 }
 
 int dxm_embed_streams(float* X, const void* table, const int64_t* ids, int rows, int S, int W, int64_t vocab,
-                      const void* ptab, const int64_t* pos, int64_t n_pos, int f32, hipStream_t st) {
+                      const void* ptab, const int64_t* pos, int64_t n_pos, float scale, int f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (ptab && !pos) return 1;
   DISPATCH_T(f32, hipLaunchKernelGGL(embed_streams_kernel<T>, dim3(rows), dim3(kThreads), 0, st, X, (const T*)table,
-                                     ids, S, W, vocab, (const T*)ptab, pos, n_pos));
+                                     ids, S, W, vocab, (const T*)ptab, pos, n_pos, scale));
   DX_CHECK_LAUNCH();
   return 0;
 }
@@ -617,12 +714,42 @@ int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int6
   return 0;
 }
 
-int dxm_diff_combine(void* out, const float* a, int64_t n_vec, int dv, float lam, float post, float eps, int f32,
+int dxm_depth_mix(float* dst, const float* stack, int64_t plane, int n, const float* w, const int64_t* rows, int n_rows,
+                  float eps, const float* nw, void* out, int W, int f32, hipStream_t st) {
+  if (n_rows <= 0) return 0;
+  if (n < 1 || W < 1 || !dst || !stack || !w || (out && !nw)) return 1;
+  const int esz = f32 ? 4 : 2;
+  auto al = [&](const void* p, int by) { return (uintptr_t)p % by == 0; };
+  const bool vec = W % 4 == 0 && plane % 4 == 0 && al(dst, 16) && al(stack, 16) && al(nw, 16) && al(out, 4 * esz);
+  if (vec) {
+    DISPATCH_T(f32, hipLaunchKernelGGL((depth_mix_kernel<T, 4>), dim3(n_rows), dim3(kThreads), 0, st, dst, stack, plane,
+                                       n, w, rows, eps, nw, (T*)out, W));
+  } else {
+    DISPATCH_T(f32, hipLaunchKernelGGL((depth_mix_kernel<T, 1>), dim3(n_rows), dim3(kThreads), 0, st, dst, stack, plane,
+                                       n, w, rows, eps, nw, (T*)out, W));
+  }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_section_norm(void* out, const void* x, int64_t x_stride, const float* w, int rows, int n, float eps, int f32,
                      hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (n < 1 || !out || !x) return 1;
+  const int blocks = (rows + kThreads / 64 - 1) / (kThreads / 64);
+  DISPATCH_T(f32, hipLaunchKernelGGL(section_norm_kernel<T>, dim3(blocks), dim3(kThreads), 0, st, (T*)out, (const T*)x,
+                                     x_stride, w, rows, n, eps));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_diff_combine(void* out, const float* a, int64_t n_vec, int dv, float lam, float post, float eps,
+                     const void* gate, int64_t gate_stride, int H, int f32, hipStream_t st) {
   if (n_vec <= 0) return 0;
+  if (gate && (H < 1 || n_vec % H)) return 1;
   const int64_t blocks = (n_vec + kThreads / 64 - 1) / (kThreads / 64);
   DISPATCH_T(f32, hipLaunchKernelGGL(diff_combine_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, st, (T*)out, a,
-                                     n_vec, dv, lam, post, eps));
+                                     n_vec, dv, lam, post, eps, (const T*)gate, gate_stride, H > 0 ? H : 1));
   DX_CHECK_LAUNCH();
   return 0;
 }

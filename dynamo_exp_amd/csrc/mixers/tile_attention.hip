@@ -22,8 +22,14 @@
 // log2 units (tanh from one exp2 and one reciprocal, the logarithm as v_log).
 //
 // Masks are evaluated per element in sequence positions: causal, sliding
-// window (p - size < j <= p) and chunked (floor(j / size) == floor(p / size)),
-// so a prompt cut anywhere gives the same result as one cut nowhere.
+// window (p - size < j <= p; with `keep` > 0 also the sequence's first `keep`
+// keys, j < keep) and chunked (floor(j / size) == floor(p / size)), so a prompt
+// cut anywhere gives the same result as one cut nowhere.  Key tiles run over
+// one numbering u of the keys a row block can see: the kept first nf keys
+// (positions 0 .. nf - 1), then the positions from the window's start on
+// (position u + shift); without kept keys nf = 0 and u + shift is the position.
+// With `sink` (a number per query vector) exp(sink) joins a softmax's
+// denominator once: a key without a value, neither scaled nor masked.
 #include "../kernels/common.h"
 
 namespace {
@@ -54,6 +60,8 @@ struct TileArgs {
   const float* hbias;  // [n_qh] (sigmoid weights only; a constant per head leaves a softmax unchanged)
   const bf16_t* gate;  // [rows, gate_stride] logits per head: the result is multiplied by their sigmoid
   int64_t gate_stride;
+  int keep;           // window mask: the first `keep` keys of a sequence stay visible (0: none)
+  const float* sink;  // [n_qh], softmax only (null: none)
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -100,12 +108,14 @@ struct TileStage {
 
   template <bool DoK = true, bool DoV = true>
   __device__ __forceinline__ void fetch(const bf16_t* kc, const bf16_t* vc, const int* bt, int bs, int Wk, int Wv,
-                                        int kt, int hi, int tid) {
+                                        int u0, int nf, int shift, int hi, int tid) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
     // One block-table lookup per lane (key kt + lane), handed to the lanes that load
     // the key by a cross-lane read: a lookup per 16-byte load would put a dependent
     // global round trip in front of each of them, and the loads retire in order.
-    const int mine = kt + (tid & 63) <= hi ? (int)slot_of(bt, bs, kt + (tid & 63)) : -1;
+    // (key u0 + lane of the visible keys' numbering: position u below nf, u + shift from there on)
+    const int ku = u0 + (tid & 63), kp = ku < nf ? ku : ku + shift;
+    const int mine = kp <= hi ? (int)slot_of(bt, bs, kp) : -1;
 #pragma unroll
     for (int i = 0; i < (DoK ? kPer : 0); ++i) {
       const int it = tid + i * NT;
@@ -193,7 +203,9 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
   const bf16_t* kc = a.kc + (int64_t)(g * a.maps + m) * d;
   const bf16_t* vc = a.vc + (int64_t)g * dv;
   const int hi = p0 + n - 1;
-  const int kt0 = first_visible(p0, a.mask, a.size) / kKeys * kKeys;
+  const int lo0 = first_visible(p0, a.mask, a.size) / kKeys * kKeys;
+  const int nf = a.mask == 1 && a.keep > 0 ? (a.keep < lo0 ? a.keep : lo0) : 0;
+  const int shift = lo0 - nf, u_end = hi - shift;
 
   // this wave's query fragments and per-row constants
   i16x4 qf[2][DB];
@@ -232,11 +244,15 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   TileStage<d, dv, 256> stage;
-  stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt0, hi, tid);
-  for (int kt = kt0; kt <= hi; kt += kKeys) {
+  stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, 0, nf, shift, hi, tid);
+  for (int ut = 0; ut <= u_end; ut += kKeys) {
+    // a tile that holds both kept first keys and window keys maps its keys one by one
+    const bool strad = ut < nf && ut + kKeys > nf;
+    const int kt = ut >= nf ? ut + shift : ut;
+    auto kpos = [&](int off) { return strad && ut + off >= nf ? kt + off + shift : kt + off; };
     stage.commit(Ks, Vt, tid);
     __syncthreads();
-    if (kt + kKeys <= hi) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, hi, tid);
+    if (ut + kKeys <= u_end) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, ut + kKeys, nf, shift, hi, tid);
     if (wave_on) {
       f32x4 S[2][4];
 #pragma unroll
@@ -269,15 +285,15 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
               float s2 = S[qb][kb][i] * a.scale;
               s2 = cap > 0.f ? capped_log2(s2, cap, inv_cap) : s2 * kLog2e;
               if (a.r1) {
-                const int dist = prow[qb] - (kt + kb * 16 + 4 * g4 + i);
+                const int dist = prow[qb] - kpos(kb * 16 + 4 * g4 + i);
                 s2 -= r1 * __builtin_amdgcn_logf(1.f + r2 * (float)(dist > 0 ? dist : 0));
               }
               S[qb][kb][i] = s2;
             }
       }
       // a tile every row of the wave sees whole needs no per-element mask
-      const bool full = 32 * w + 31 < n && kt + kKeys - 1 <= p0 + 32 * w &&
-                        kt >= first_visible(p0 + 32 * w + 31, a.mask, a.size);
+      const bool full = 32 * w + 31 < n && !strad && kt + kKeys - 1 <= p0 + 32 * w &&
+                        (ut + kKeys <= nf || kt >= first_visible(p0 + 32 * w + 31, a.mask, a.size));
       i16x4 Ph[2][4], Pl[2][4];
       if (a.wfn) {
         // sigmoid weights: w = 1 / (1 + 2^-(x log2 e)), x = s + hbias; invisible keys weigh 0;
@@ -290,8 +306,8 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
             float p[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              const int kj = kt + kb * 16 + 4 * g4 + i;
-              const bool vis = full || (okrow[qb] && kj >= lrow[qb] && kj <= prow[qb]);
+              const int kj = kpos(kb * 16 + 4 * g4 + i);
+              const bool vis = full || (okrow[qb] && (kj >= lrow[qb] || kj < a.keep) && kj <= prow[qb]);
               const float w_ = __builtin_amdgcn_rcpf(1.f + fast_exp2(-fmaf(S[qb][kb][i], xs, hb2)));
               p[i] = vis ? w_ : 0.f;
             }
@@ -319,8 +335,8 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
           for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              const int kj = kt + kb * 16 + 4 * g4 + i;
-              const bool vis = okrow[qb] && kj >= lrow[qb] && kj <= prow[qb];
+              const int kj = kpos(kb * 16 + 4 * g4 + i);
+              const bool vis = okrow[qb] && (kj >= lrow[qb] || kj < a.keep) && kj <= prow[qb];
               const float s = vis ? S[qb][kb][i] : -INFINITY;
               S[qb][kb][i] = s;
               mloc = fmaxf(mloc, s);
@@ -388,6 +404,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
     l += __shfl_xor(l, 32, 64);
     if (!okrow[qb]) continue;
     const int r = 32 * w + 16 * qb + c16;
+    if (a.sink && !a.wfn) l += fast_exp2(a.sink[qh] * kLog2e - mx[qb]);  // mx in log2 units, finite: a row sees itself
     float inv = a.wfn ? 1.f : 1.f / l;
     if (a.gate) inv /= 1.f + __expf(-bf16_to_f32(a.gate[(int64_t)(row0 + r) * a.gate_stride + head]));
     OutT* o = (OutT*)a.out + ((int64_t)(row0 + r) * a.n_qh + qh) * dv + 4 * g4;
@@ -423,6 +440,7 @@ struct GroupArgs {
   const float* r2;
   int wfn;
   const float* hbias;
+  int keep;  // window mask: the first `keep` keys of a sequence stay visible (0: none)
 };
 
 template <int DB, int DVB, int QB>
@@ -440,7 +458,10 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   const bf16_t* kc = a.kc + (int64_t)gm * d;
   const bf16_t* vc = a.vc + (int64_t)g * dv;
   const int lo = first_visible(p, a.mask, a.size);
-  const int tiles = (p - lo + kKeys) / kKeys;
+  // the visible keys in one numbering: the kept first nf keys, then lo .. p (position u + shift)
+  const int nf = a.mask == 1 && a.keep > 0 ? (a.keep < lo ? a.keep : lo) : 0;
+  const int shift = lo - nf;
+  const int tiles = (nf + p - lo + kKeys) / kKeys;
   const int tpp = (tiles + a.parts - 1) / a.parts;
   const int t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
 
@@ -475,19 +496,19 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   // accumulators, so K and V are staged one after the other and nothing is prefetched
   constexpr bool kWide = DB + DVB > 16;
   TileStage<d, dv, 64> stage;
-  if (!kWide && t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, lo + t0 * kKeys, p, lane);
+  if (!kWide && t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, t0 * kKeys, nf, shift, p, lane);
   for (int t = t0; t < t1; ++t) {
-    const int kt = lo + t * kKeys;
+    const int ut = t * kKeys;
     if constexpr (kWide) {
-      stage.template fetch<true, false>(kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+      stage.template fetch<true, false>(kc, vc, bt, a.bs, a.Wk, a.Wv, ut, nf, shift, p, lane);
       stage.template commit<true, false>(Ks, Vt, lane);
-      stage.template fetch<false, true>(kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+      stage.template fetch<false, true>(kc, vc, bt, a.bs, a.Wk, a.Wv, ut, nf, shift, p, lane);
       stage.template commit<false, true>(Ks, Vt, lane);
     } else {
       stage.commit(Ks, Vt, lane);
     }
     __syncthreads();
-    if (!kWide && t + 1 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, p, lane);
+    if (!kWide && t + 1 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, ut + kKeys, nf, shift, p, lane);
     f32x4 S[QB][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -509,7 +530,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int kj = kt + kb * 16 + 4 * g4 + i;
+          const int ku = ut + kb * 16 + 4 * g4 + i, kj = ku < nf ? ku : ku + shift;
           float s = S[qb][kb][i] * a.scale;
           if (cap > 0.f) s = cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * s * inv_cap)));
           if (a.r1) s -= r1[qb] * __logf(1.f + r2[qb] * (float)(p - kj > 0 ? p - kj : 0));
@@ -630,7 +651,7 @@ extern "C" {
 
 // 1 when tile_attention has an instance for the head widths
 int dxm_tile_attention_ok(int d, int dv) {
-  const int pairs[][2] = {{2, 2}, {3, 3}, {3, 6}, {4, 4}, {4, 8}, {8, 8}, {8, 16}, {16, 16}};
+  const int pairs[][2] = {{2, 2}, {2, 4}, {3, 3}, {3, 6}, {4, 4}, {4, 8}, {8, 8}, {8, 16}, {9, 8}, {16, 12}, {16, 16}};
   for (auto& p : pairs)
     if (d == p[0] * 16 && dv == p[1] * 16) return 1;
   return 0;
@@ -640,22 +661,25 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
                        const int* seq, const int* bt, int bt_stride, int bs, const int* tiles, int n_tiles, int n_qh,
                        int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask, int size,
                        float softcap, const float* r1, const float* r2, int wfn, const float* hbias, const void* gate,
-                       int64_t gate_stride, int out_f32, hipStream_t st) {
+                       int64_t gate_stride, int keep, const float* sink, int out_f32, hipStream_t st) {
   if (n_tiles <= 0) return 0;
-  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1 || keep < 0 || (keep && mask != 1)) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || !(scale > 0.f)) return 3;
   if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 8) return 4;
   TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
              tiles, n_qh, maps, group, Wk, Wv, scale, mask, size, softcap, r1, r2, wfn, hbias, (const bf16_t*)gate,
-             gate_stride};
+             gate_stride, keep, sink};
   TILE_CASE(2, 2)
+  TILE_CASE(2, 4)
   TILE_CASE(3, 3)
   TILE_CASE(3, 6)
   TILE_CASE(4, 4)
   TILE_CASE(4, 8)
   TILE_CASE(8, 8)
   TILE_CASE(8, 16)
+  TILE_CASE(9, 8)
+  TILE_CASE(16, 12)
   TILE_CASE(16, 16)
   return 2;
 }
@@ -668,21 +692,24 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
 int dxm_group_decode(float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
                      const int* seq, const int* bt, int bt_stride, int bs, int rows, int n_qh, int maps, int group,
                      int d, int dv, int Wk, int Wv, float scale, int mask, int size, float softcap, const float* r1,
-                     const float* r2, int wfn, const float* hbias, int parts, hipStream_t st) {
+                     const float* r2, int wfn, const float* hbias, int keep, int parts, hipStream_t st) {
   if (rows <= 0) return 0;
-  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1) return 6;
+  if (softcap < 0.f || (r1 && !r2) || wfn < 0 || wfn > 1 || keep < 0 || (keep && mask != 1)) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || rows > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535) return 3;
   if (!ws || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
   GroupArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, ws, pos, seq, bt, bt_stride, bs,
-              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias};
+              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts, softcap, r1, r2, wfn, hbias, keep};
   GROUP_CASE(2, 2)
+  GROUP_CASE(2, 4)
   GROUP_CASE(3, 3)
   GROUP_CASE(3, 6)
   GROUP_CASE(4, 4)
   GROUP_CASE(4, 8)
   GROUP_CASE(8, 8)
   GROUP_CASE(8, 16)
+  GROUP_CASE(9, 8)
+  GROUP_CASE(16, 12)
   GROUP_CASE(16, 16)
   return 2;
 }

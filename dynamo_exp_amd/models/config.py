@@ -150,6 +150,9 @@ class LayeredConfig:
     streams: int | None = None  # parallel residual streams (None: one plain residual)
     token_side: dict | None = None  # {"dim"}: per-layer token input (a slice of a second embedding per layer)
     learned_positions: bool = False  # a learned vector per position is added to the embedding
+    embedding_scale: float = 1.0  # the embedding row is multiplied by this
+    logit_scale: float = 1.0  # the logits are multiplied by this
+    canon: dict | None = None  # {"taps"}: a short causal convolution over time on every mixer's input
     max_position_embeddings: int = 1 << 20
     tie_word_embeddings: bool = False
     bos_token_id: int = 0
@@ -179,6 +182,8 @@ class LayeredConfig:
             return n + self._bolinex_params()
         if self.architecture == "Nefivik":
             return n + self._nefivik_params()
+        if self.architecture == "Sobivik":
+            return n - W + 1 + self._sobivik_params()
         for L in self.layers:
             m, t = L["mixer"], L["type"]
             H, d, dv = m["heads"], m["dim"], m["vdim"]
@@ -237,6 +242,26 @@ class LayeredConfig:
             n += 2 * W * side + (W if side else 0)
         return n
 
+    def _sobivik_params(self) -> int:
+        W = self.hidden_size
+        taps = int((self.canon or {}).get("taps", 0))
+        n = 0
+        for i, L in enumerate(self.layers):
+            m = L["mixer"]
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            n += 4 + W * taps + i + 2  # scalar norms, input convolution, depth weights
+            if L["type"] == "retention":
+                n += (2 * H * d + 2 * H * dv) * W + W * H * dv
+            elif L["type"] == "latent_attention":
+                r, qr, dr = m["kv_rank"], m["q_rank"], m["rot_dim"]
+                n += qr * (W + 1) + H * (d + dr) * qr + (r + dr) * W + r + H * (d + dv) * r + H + 2 * H * dv * W
+            else:
+                G = m["kv_heads"]
+                n += (2 * H * d + 2 * G * d + G * dv + H) * W + 4 * d + W * H * dv
+            if L.get("mlp"):
+                n += 3 * W * L["mlp"]["ff"]
+        return n
+
     def to_dict(self) -> dict:
         return dataclasses.asdict(self)
 
@@ -248,6 +273,8 @@ class LayeredConfig:
                    layers=list(c["layers"]), loop=c.get("loop"), rms_norm_eps=float(c["norm"]["eps"]),
                    streams=c.get("streams"), token_side=c.get("token_side"),
                    learned_positions="max_positions" in c,
+                   embedding_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                   logit_scale=float(c.get("logit_scale", 1.0)), canon=c.get("canon"),
                    max_position_embeddings=int(maxpos) if maxpos else 1 << 20,
                    eos_token_id=list(c.get("eos_token_id", [])))
 
@@ -263,12 +290,18 @@ class LayeredConfig:
             d["token_side"] = self.token_side
         if self.learned_positions:
             d["max_positions"] = self.max_position_embeddings
+        if self.embedding_scale != 1.0:
+            d["embedding"] = {"scale": self.embedding_scale}
+        if self.logit_scale != 1.0:
+            d["logit_scale"] = self.logit_scale
+        if self.canon:
+            d["canon"] = self.canon
         with open(os.path.join(path, "config.json"), "w") as f:
             json.dump(d, f, indent=1)
 
 
 # config.json `architecture` values served by LayeredConfig
-LAYERED_ARCHITECTURES = ("Bekulix", "Bolinex", "Nefivik")
+LAYERED_ARCHITECTURES = ("Bekulix", "Bolinex", "Nefivik", "Sobivik")
 
 
 def _bekulix_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, window, chunk, vocab=32000, streams=4):
@@ -334,6 +367,28 @@ def _nefivik_preset(name, W, n_layers, heads, kv_heads, d, window, experts, top,
         layers.append({"type": "attention", "mixer": mixer, "mlp": dict(mlp)})
     return LayeredConfig(name=name, architecture="Nefivik", vocab_size=vocab, hidden_size=W, layers=layers,
                          rms_norm_eps=1e-5, token_side={"dim": side} if side else None)
+
+
+def _sobivik_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, q_rank, rot_dim, window, keep, vocab=32000,
+                    taps=4):
+    """A Sobivik stack at a real model's layer sizes: differential attention
+    (a window that keeps the first tokens), retention and latent attention
+    (rotated key part, window, sink) layers in turn, all with a dense gated
+    feed-forward, the input convolution and the depth average."""
+    dif = {"type": "attention", "mixer": {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": d,
+                                          "vdim": 2 * d, "scale": d ** -0.5, "diff": 0.3,
+                                          "mask": {"size": window, "keep_first": keep}}}
+    ret = {"type": "retention", "mixer": {"heads": heads, "dim": d, "vdim": d,
+                                          "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(1, heads - 1)) for h in range(heads)]}}
+    lat = {"type": "latent_attention", "mixer": {
+        "heads": heads, "dim": d, "rot_dim": rot_dim, "vdim": d, "kv_rank": rank, "q_rank": q_rank,
+        "scale": (d + rot_dim) ** -0.5, "mask": {"size": window},
+        "rot": {"base": 10000.0, "dims": rot_dim, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    cyc = [dif, ret, lat]
+    layers = [{**cyc[i % 3], "mixer": dict(cyc[i % 3]["mixer"]), "mlp": {"kind": "dense", "ff": ff}}
+              for i in range(n_layers)]
+    return LayeredConfig(name=name, architecture="Sobivik", vocab_size=vocab, hidden_size=W, layers=layers,
+                         rms_norm_eps=1e-5, embedding_scale=float(W) ** 0.5, logit_scale=0.25, canon={"taps": taps})
 
 
 # CLIP ViT-L/14 at 336 px, the LLaVA-1.5 vision tower; features from the
@@ -408,6 +463,12 @@ PRESETS["nefivik-tiny"] = _nefivik_preset("nefivik-tiny", 192, 6, 3, 1, 32, 48, 
 # of the dense width, 2 chosen
 PRESETS["nefivik-8b-shapes"] = _nefivik_preset("nefivik-8b-shapes", 4096, 9, 32, 8, 128, 1024, experts=16, top=2,
                                                expert_ff=3584, groups=(4, 2), side=256, vocab=128256)
+
+
+PRESETS["sobivik-tiny"] = _sobivik_preset("sobivik-tiny", 192, 384, 6, 4, 2, 32, 64, 48, 32, 40, 6, vocab=512, taps=3)
+# Llama-3-8B's layer sizes (width 4096, ff 14336, 32 x 128 heads, 8 KV heads), 9 layers; latent rank 192 + 64 rotated
+PRESETS["sobivik-8b-shapes"] = _sobivik_preset("sobivik-8b-shapes", 4096, 14336, 9, 32, 8, 128, 192, 1536, 64, 1024,
+                                               64, vocab=128256)
 
 
 def get_config(name_or_path: str) -> ModelConfig:

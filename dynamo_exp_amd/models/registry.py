@@ -36,6 +36,12 @@ def _nefivik():
     return NefivikForCausalLM
 
 
+def _sobivik():
+    from .sobivik import SobivikForCausalLM
+
+    return SobivikForCausalLM
+
+
 # architecture -> (class loader, activation dtypes the class has kernels for)
 MODEL_REGISTRY = {
     "LlamaForCausalLM": (_llama, ("bfloat16",)),
@@ -43,6 +49,7 @@ MODEL_REGISTRY = {
     "Bekulix": (_bekulix, ("bfloat16", "float32")),
     "Bolinex": (_bolinex, ("bfloat16", "float32")),
     "Nefivik": (_nefivik, ("bfloat16", "float32")),
+    "Sobivik": (_sobivik, ("bfloat16", "float32")),
 }
 
 

@@ -64,26 +64,35 @@ def _fp32_param(t: torch.Tensor | None, name: str):
 
 # ----------------------------------------------------------------- residual streams
 def embed_streams(ids: torch.Tensor, table: torch.Tensor, n_streams: int, pos_table: torch.Tensor | None = None,
-                  positions: torch.Tensor | None = None) -> torch.Tensor:
-    """X [T, S, W] fp32 with every stream equal to table[ids], plus the learned
-    position vector pos_table[positions] when a table of them is given (the
-    sum is formed in fp32)."""
+                  positions: torch.Tensor | None = None, scale: float = 1.0,
+                  out: torch.Tensor | None = None) -> torch.Tensor:
+    """X [T, S, W] fp32 with every stream equal to table[ids] * scale, plus the
+    learned position vector pos_table[positions] when a table of them is given
+    (product and sum are formed in fp32).  out: a contiguous fp32 tensor of
+    T * S * W elements to fill instead of a new one."""
     T = ids.shape[0]
     V, W = table.shape
     if pos_table is not None and (positions is None or pos_table.shape[1] != W or pos_table.dtype != table.dtype):
         raise ValueError("embed_streams: position table of the embedding's width and dtype, with positions")
     if not table.is_cuda:
-        x = table[ids].float()
+        x = table[ids].float() * scale
         if pos_table is not None:
             x = x + pos_table[positions].float()
-        return x[:, None, :].repeat(1, n_streams, 1).contiguous()
-    X = torch.empty((T, n_streams, W), dtype=torch.float32, device=table.device)
+        x = x[:, None, :].repeat(1, n_streams, 1).contiguous()
+        if out is None:
+            return x
+        out.view(T, n_streams, W).copy_(x)
+        return out.view(T, n_streams, W)
+    if out is not None and (out.dtype != torch.float32 or not out.is_contiguous() or out.numel() != T * n_streams * W):
+        raise TypeError("embed_streams: out is contiguous float32 with T * S * W elements")
+    X = out.view(T, n_streams, W) if out is not None else \
+        torch.empty((T, n_streams, W), dtype=torch.float32, device=table.device)
     ids = ids if ids.dtype == torch.int64 else ids.long()
     if pos_table is not None and (positions.dtype != torch.int64 or not pos_table.is_contiguous()):
         raise TypeError("embed_streams: int64 positions, contiguous position table")
     _m().embed_streams(X.data_ptr(), table.data_ptr(), ids.data_ptr(), T, n_streams, W, V, _ptr(pos_table),
                        _ptr(positions) if pos_table is not None else 0,
-                       pos_table.shape[0] if pos_table is not None else 0, _f32(table), _stream())
+                       pos_table.shape[0] if pos_table is not None else 0, float(scale), _f32(table), _stream())
     return X
 
 
@@ -187,6 +196,64 @@ def stream_step(X: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | Non
     _m().stream_step(X.data_ptr(), _ptr(y), y.stride(0) if y is not None else 0, _ptr(mix), _ptr(gain), _ptr(rin),
                      _ptr(norm_w), float(eps), _ptr(out), W, T, S, W, f32, _stream())
     return out
+
+
+def section_norm(x: torch.Tensor, weight: torch.Tensor | None, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * weight over a column section x [T, n] of
+    wider rows (contiguous rows, any row stride), e.g. a low-rank latent inside
+    a fused projection's output; fp32 sums, result [T, n] in x's dtype."""
+    T, n = x.shape
+    _fp32_param(weight, "weight")
+    if x.stride(1) != 1 or (weight is not None and weight.numel() != n):
+        raise ValueError("section_norm: rows contiguous, one weight per column")
+    if not x.is_cuda:
+        xf = x.float()
+        y = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+        return (y * weight if weight is not None else y).to(x.dtype)
+    out = torch.empty((T, n), dtype=x.dtype, device=x.device)
+    _m().section_norm(out.data_ptr(), x.data_ptr(), x.stride(0), _ptr(weight), T, n, float(eps), _f32(x), _stream())
+    return out
+
+
+def depth_mix(stack: torch.Tensor, n: int, weights: torch.Tensor, dst: torch.Tensor | None = None,
+              rows: torch.Tensor | None = None, norm_w: torch.Tensor | None = None, eps: float = 1e-6,
+              out_dtype: torch.dtype = torch.bfloat16):
+    """A weighted sum over depth: stack [>= n, T, W] fp32 holds one [T, W]
+    plane per layer result (plane 0 the embedding output);
+        x[r] = sum_{j < n} weights[j] * stack[j, rows[r]]        (rows None: every row)
+    in fp32, summed in the order j = 0, 1, ....  x is written to dst (fp32
+    [len(rows) or T, W]; a later plane of the stack is the usual choice, so the
+    next layer updates it in place into its own result) and returned together
+    with norm(x) = x / sqrt(mean(x^2) + eps) * norm_w in out_dtype (None without
+    norm_w)."""
+    if stack.dim() != 3 or stack.dtype != torch.float32 or not stack.is_contiguous() or not 1 <= n <= stack.shape[0]:
+        raise TypeError("depth_mix: stack is contiguous float32 [planes, T, W] with n <= planes")
+    _, T, W = stack.shape
+    _fp32_param(weights, "weights")
+    _fp32_param(norm_w, "norm_w")
+    if weights.numel() != n or (norm_w is not None and norm_w.numel() != W):
+        raise ValueError("depth_mix: one weight per plane, one norm weight per column")
+    R = T if rows is None else rows.numel()
+    if dst is None:
+        dst = torch.empty((R, W), dtype=torch.float32, device=stack.device)
+    if dst.shape != (R, W) or dst.dtype != torch.float32 or not dst.is_contiguous():
+        raise TypeError("depth_mix: dst is contiguous float32 [rows, W]")
+    if not stack.is_cuda:
+        src = stack[:n] if rows is None else stack[:n, rows.long()]
+        x = torch.zeros((R, W), dtype=torch.float32)
+        for j in range(n):
+            x += weights[j] * src[j]
+        dst.copy_(x)
+        h = None
+        if norm_w is not None:
+            h = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * norm_w).to(out_dtype)
+        return dst, h
+    if rows is not None and (rows.dtype != torch.int64 or not rows.is_contiguous()):
+        raise TypeError("depth_mix: rows must be contiguous int64")
+    h = torch.empty((R, W), dtype=out_dtype, device=stack.device) if norm_w is not None else None
+    _m().depth_mix(dst.data_ptr(), stack.data_ptr(), T * W, n, weights.data_ptr(), _ptr(rows), R, float(eps),
+                   _ptr(norm_w), _ptr(h), W, int(out_dtype == torch.float32), _stream())
+    return dst, h
 
 
 # ----------------------------------------------------------------- feed-forward
@@ -336,7 +403,8 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
               group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
               out_f32: bool = False, tiles: torch.Tensor | None = None, n_tile_rows: int = 0, softcap: float = 0.0,
               dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None, weights: str = "softmax",
-              head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None) -> torch.Tensor:
+              head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None, keep_first: int = 0,
+              sink: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of one step's rows: the first n_tile_rows rows (prompt chunks,
     cut into `tiles` [n, 2] = first row, row count) on the matrix-core prefill
     kernel where it applies, all other rows (decode tokens; every row when it
@@ -345,9 +413,11 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     T = q.shape[0]
     if not tile_attention_ok(q, d, dv) or not scale > 0:  # the matrix-core kernels fold a positive scale
         return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
-                             mask, size, parts, out_f32, softcap, dist_bias, weights, head_bias, head_gate)
+                             mask, size, parts, out_f32, softcap, dist_bias, weights, head_bias, head_gate, keep_first,
+                             sink)
     _check_score_terms(softcap, dist_bias, n_qh)
     _check_weight_terms(weights, head_bias, head_gate, q, n_qh, maps)
+    _check_mask_terms(mask, keep_first, sink, weights, n_qh)
     if tiles is None:
         n_tile_rows = 0
     if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous() or \
@@ -372,15 +442,15 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
             raise TypeError("attention: prompt-chunk rows need seq and int32 tiles")
         _m().tile_attention(out.data_ptr(), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
                             positions.data_ptr(), seq.data_ptr(), *common, tiles.data_ptr(), tiles.shape[0], *heads,
-                            _ptr(head_gate), gs, int(out_f32), _stream())
+                            _ptr(head_gate), gs, int(keep_first), _ptr(sink), int(out_f32), _stream())
     n_dec = T - n_tile_rows
     if n_dec:  # decode rows: the heads of a K/V group share one wave's key tiles
         r0 = n_tile_rows
         ws = torch.empty((n_dec, n_qh, parts, 2 + dv), dtype=torch.float32, device=q.device)
         _m().group_decode(out[r0:].data_ptr(), ws.data_ptr(), q[r0:].data_ptr(), q.stride(0), kc.data_ptr(),
                           vc.data_ptr(), positions[r0:].data_ptr(), _ptr(seq[r0:] if seq is not None else None),
-                          *common, n_dec, *heads, _ptr(head_gate[r0:]) if head_gate is not None else 0, gs, parts,
-                          int(out_f32), _stream())
+                          *common, n_dec, *heads, _ptr(head_gate[r0:]) if head_gate is not None else 0, gs,
+                          int(keep_first), _ptr(sink), parts, int(out_f32), _stream())
     return out
 
 
@@ -392,6 +462,14 @@ def _check_score_terms(softcap: float, dist_bias, n_qh: int) -> None:
             _fp32_param(t, "dist_bias")
             if t.numel() != n_qh:
                 raise ValueError("dist_bias: one (r1, r2) pair per query vector")
+
+
+def _check_mask_terms(mask: str, keep_first: int, sink, weights: str, n_qh: int) -> None:
+    if keep_first < 0 or (keep_first and mask != "window"):
+        raise ValueError("keep_first: a count of first keys that a window mask keeps visible")
+    _fp32_param(sink, "sink")
+    if sink is not None and (sink.numel() != n_qh or weights != "softmax"):
+        raise ValueError("sink: one number per query vector, with softmax weights")
 
 
 def _check_weight_terms(weights: str, head_bias, head_gate, q: torch.Tensor, n_qh: int, maps: int) -> None:
@@ -410,7 +488,8 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
                   group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
                   out_f32: bool = False, softcap: float = 0.0,
                   dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None, weights: str = "softmax",
-                  head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None) -> torch.Tensor:
+                  head_bias: torch.Tensor | None = None, head_gate: torch.Tensor | None = None, keep_first: int = 0,
+                  sink: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of T rows over their sequences' paged caches.
     q [T, >= n_qh * d] (n_qh = heads * maps query vectors per row); returns
     [T, n_qh, dv].  Query vector qh reads K head (qh // maps // group) * maps +
@@ -422,10 +501,15 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
     keys' weights are softmax(s); 'sigmoid': every visible key weighs
     sigmoid(s), not normalised over the keys.  With head_gate [T, heads]
     (logits, a column section) head h's result is multiplied by
-    sigmoid(head_gate[:, h])."""
+    sigmoid(head_gate[:, h]).  Masks: 'causal' j <= i; 'window' also
+    i - j < size, or j < keep_first (the sequence's first keep_first keys stay
+    visible at their true positions); 'chunk' floor(j / size) = floor(i / size).
+    With sink (fp32 [n_qh]) the softmax denominator also holds exp(sink[qh]):
+    a key without a value, neither scaled nor masked, counted once."""
     T = q.shape[0]
     _check_score_terms(softcap, dist_bias, n_qh)
     _check_weight_terms(weights, head_bias, head_gate, q, n_qh, maps)
+    _check_mask_terms(mask, keep_first, sink, weights, n_qh)
     if mask not in MASKS:
         raise ValueError(f"unknown mask {mask!r}")
     if mask != "causal" and size < 1:
@@ -460,9 +544,16 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
                 sc = sc - dist_bias[0][:, None, None] * torch.log1p(dist_bias[1][:, None, None] * dist[None])
             if head_bias is not None:
                 sc = sc + head_bias[:, None, None]
-            vis = (j[None, :] <= p[:, None]) & (j[None, :] >= first_visible(p, mask, size)[:, None])
+            near = j[None, :] >= first_visible(p, mask, size)[:, None]
+            if keep_first:
+                near = near | (j[None, :] < keep_first)
+            vis = (j[None, :] <= p[:, None]) & near
             sc = sc.masked_fill(~vis[None], float("-inf"))
-            wt = torch.softmax(sc, -1) if weights == "softmax" else torch.sigmoid(sc)
+            if weights == "softmax" and sink is not None:
+                sc = torch.cat([sc, sink.view(n_qh, 1, 1).expand(n_qh, sc.shape[1], 1)], -1)
+                wt = torch.softmax(sc, -1)[..., :n]
+            else:
+                wt = torch.softmax(sc, -1) if weights == "softmax" else torch.sigmoid(sc)
             out[rows] = torch.einsum("hij,jhd->ihd", wt, V)
         if head_gate is not None:
             out = out * torch.sigmoid(head_gate.float()).repeat_interleave(maps, 1)[:, :, None]
@@ -481,22 +572,32 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
                        T, n_qh, maps, group, d, dv, Wk, Wv, float(scale), MASKS[mask], int(size), float(softcap),
                        _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0,
                        WEIGHTS[weights], _ptr(head_bias), _ptr(head_gate),
-                       head_gate.stride(0) if head_gate is not None else 0, parts, _f32(q),
+                       head_gate.stride(0) if head_gate is not None else 0, int(keep_first), _ptr(sink), parts, _f32(q),
                        int(odt == torch.float32), _stream())
     return out
 
 
-def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, out_dtype: torch.dtype,
+                 head_gate: torch.Tensor | None = None) -> torch.Tensor:
     """a [T, H, 2, dv] fp32 (two maps' outputs) -> [T, H * dv]:
-    unit_rms_over_dv(a1 - lam * a2) * post."""
+    unit_rms_over_dv(a1 - lam * a2) * post; with head_gate [T, H] (logits, a
+    column section of out_dtype) head h is then multiplied by
+    sigmoid(head_gate[:, h]) -- after the unit norm, which would cancel a gate
+    applied to the maps."""
     T, H, two, dv = a.shape
     if two != 2 or a.dtype != torch.float32 or not a.is_contiguous():
         raise TypeError("diff_combine: a must be contiguous float32 [T, H, 2, dv]")
+    if head_gate is not None and (head_gate.shape != (T, H) or head_gate.stride(1) != 1 or
+                                  head_gate.dtype != out_dtype):
+        raise ValueError("diff_combine: head_gate is [T, H] of the output dtype with contiguous rows")
     if not a.is_cuda:
         o = a[:, :, 0] - lam * a[:, :, 1]
         o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * post
+        if head_gate is not None:
+            o = o * torch.sigmoid(head_gate.float())[:, :, None]
         return o.reshape(T, H * dv).to(out_dtype)
     out = torch.empty((T, H * dv), dtype=out_dtype, device=a.device)
-    _m().diff_combine(out.data_ptr(), a.data_ptr(), T * H, dv, float(lam), float(post), float(eps),
-                      int(out_dtype == torch.float32), _stream())
+    _m().diff_combine(out.data_ptr(), a.data_ptr(), T * H, dv, float(lam), float(post), float(eps), _ptr(head_gate),
+                      head_gate.stride(0) if head_gate is not None else 0, H, int(out_dtype == torch.float32),
+                      _stream())
     return out

@@ -1,5 +1,5 @@
 """Ops with per-sequence state: the generalized delta rule (a running matrix
-per head), short causal convolutions over time fused with rotary positions and
+per head), retention (a running matrix with a fixed decay per head), short causal convolutions over time fused with rotary positions and
 the paged cache write, and the per-head unit-RMS + gate that follows a
 recurrent mixer.
 
@@ -55,6 +55,83 @@ def rotary_frequencies(dims: int, base: float, scaling: dict | None = None) -> t
                 f = (1.0 - s) * f / fac + s * f
         out.append(f)
     return torch.tensor(out, dtype=torch.float64).to(torch.float32)
+
+
+def yarn_frequencies(dims: int, base: float, scaling: dict | None = None) -> tuple[torch.Tensor, float]:
+    """(f [dims / 2] fp32, mag): f_i = base^(-2 i / dims), and with scaling =
+    {factor, original, fast, slow} (YaRN) the blend
+        f_i / factor * ramp_i + f_i * (1 - ramp_i),   ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+    between the dimensions lo = max(floor(dim(fast)), 0) and hi = min(ceil(dim(slow)), dims - 1), where
+    dim(t) = dims * ln(original / (2 pi t)) / (2 ln base) is the dimension whose wavelength fits t
+    times into the original length; mag = 0.1 ln(factor) + 1 multiplies cosines and sines
+    (1 without scaling).  Computed in float64."""
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    mag = 1.0
+    if scaling:
+        fac, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def dim_of(turns: float) -> float:
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+        lo = max(math.floor(dim_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(dim_of(float(scaling["slow"]))), dims - 1)
+        for i in range(dims // 2):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f[i] = f[i] / fac * ramp + f[i] * (1.0 - ramp)
+        mag = 0.1 * math.log(fac) + 1.0
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32), mag
+
+
+def latent_rope(qa: torch.Tensor, q: torch.Tensor, q_head: int, q_off: int, kv: torch.Tensor, r: int, dr: int,
+                norm_w: torch.Tensor, eps: float, inv_freq: torch.Tensor | None, mag: float,
+                positions: torch.Tensor, kv_slots: torch.Tensor, cache: torch.Tensor) -> torch.Tensor:
+    """Query / key preparation of latent attention with a rotated key part.
+    Per token row t: the latent kv[t, :r] is RMS-normed (weight norm_w) into
+    cache[slot, :r]; the key part kv[t, r:r + dr], shared by all heads and not
+    normed, is rotated into cache[slot, r:]; and head h's query is assembled
+    as [qa[h, t] (r) | rotate(q[t, h * q_head + q_off : + dr])] -- qa [H, T, r]
+    is the head's unrotated query part already times the head's key
+    up-projection.  Returns q' [T, H * (r + dr)].  Rotation: the first
+    2 len(inv_freq) columns of a part, column i paired with i + len(inv_freq),
+    by the angle position * inv_freq[i], cosines and sines times mag; the rest
+    pass unchanged.  Rows with slot < 0 cache nothing."""
+    H, T, _ = qa.shape
+    half = 0 if inv_freq is None else inv_freq.numel()
+    _fp32_param(norm_w, "norm_w")
+    _fp32_param(inv_freq, "inv_freq")
+    Wc = r + dr
+    if qa.shape != (H, T, r) or not qa.is_contiguous() or kv.shape[0] != T or kv.shape[1] < Wc or kv.stride(1) != 1 or \
+            q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < (H - 1) * q_head + q_off + dr or 2 * half > dr or \
+            q_off + dr > q_head or norm_w.numel() != r:
+        raise ValueError("latent_rope: sections do not fit the rows")
+    if cache.shape[-1] != Wc or not cache.is_contiguous() or any(t.dtype != qa.dtype for t in (q, kv, cache)):
+        raise ValueError("latent_rope: cache rows are [latent | rotated key] of the activation dtype")
+    if not qa.is_cuda:
+        def rot(x):  # [T, ..., dr]
+            if not half:
+                return x
+            ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+            shape = [T] + [1] * (x.dim() - 2) + [half]
+            c, s_ = (torch.cos(ang) * mag).view(shape), (torch.sin(ang) * mag).view(shape)
+            a_, b_ = x[..., :half], x[..., half:2 * half]
+            return torch.cat([a_ * c - b_ * s_, b_ * c + a_ * s_, x[..., 2 * half:]], -1)
+
+        kvf = kv.float()
+        c = kvf[:, :r]
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w
+        row = torch.cat([c, rot(kvf[:, r:Wc])], -1).to(cache.dtype)
+        ok = kv_slots >= 0
+        cache[kv_slots[ok]] = row[ok]
+        qr = torch.stack([q[:, h * q_head + q_off:h * q_head + q_off + dr] for h in range(H)], 1).float()
+        out = torch.cat([qa.transpose(0, 1).float(), rot(qr)], -1).to(qa.dtype)
+        return out.reshape(T, H * Wc)
+    if positions.dtype != torch.int64 or kv_slots.dtype != torch.int64:
+        raise TypeError("latent_rope: int64 positions and kv_slots")
+    out = torch.empty((T, H * Wc), dtype=qa.dtype, device=qa.device)
+    _m().latent_rope(out.data_ptr(), qa.data_ptr(), q.data_ptr(), q.stride(0), q_head, q_off, kv.data_ptr(),
+                     kv.stride(0), norm_w.data_ptr(), float(eps), _ptr(inv_freq), half, float(mag),
+                     positions.data_ptr(), kv_slots.data_ptr(), cache.data_ptr(), T, H, r, dr, _f32(qa), _stream())
+    return out
 
 
 # ----------------------------------------------------------------- short convolution + rotary + cache write
@@ -224,11 +301,62 @@ def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tenso
     return out
 
 
+def retention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, k_scale: float,
+              state: torch.Tensor, positions: torch.Tensor, seq_rows: torch.Tensor | None, state_slots: torch.Tensor,
+              n_heads: int, dk: int, dv: int) -> torch.Tensor:
+    """Retention (linear attention with a fixed decay per head, no softmax and
+    no denominator) over the rows of a step, per sequence and head from the
+    sequence's state S [dk, dv] (fp32; stored column by column, state
+    [slots, H, dv, dk] with state[s, h, j, i] = S[i, j]; updated in place):
+        S_t = decay[h] S_(t-1) + (k_scale k_t) v_t^T,     o_t = S_t^T q_t.
+    q, k [T, H dk] and v [T, H dv] are column sections (contiguous rows, any
+    row stride) of projection outputs; decay fp32 [H].  Returns o [T, H dv]
+    fp32.  Everything but reading the inputs is fp32."""
+    T = q.shape[0]
+    n_seq = state_slots.numel()
+    _fp32_param(decay, "decay")
+    _check_step(positions, seq_rows, state_slots)
+    for t, wd in ((q, dk), (k, dk), (v, dv)):
+        if t.shape != (T, n_heads * wd) or t.stride(1) != 1 or t.dtype != q.dtype:
+            raise ValueError("retention: q, k [T, H dk] and v [T, H dv] with contiguous rows, one dtype")
+    if state.shape[1:] != (n_heads, dv, dk) or state.dtype != torch.float32 or not state.is_contiguous() or \
+            decay.numel() != n_heads:
+        raise ValueError("retention: state is contiguous float32 [slots, H, dv, dk], decay [H]")
+    if not q.is_cuda:
+        H = n_heads
+        out = torch.zeros((T, H, dv), dtype=torch.float32)
+        qf, kf, vf = q.float().view(T, H, dk), k.float().view(T, H, dk) * k_scale, v.float().view(T, H, dv)
+        b = _seq_bounds(seq_rows, n_seq)
+        for s in range(n_seq):
+            r0, r1 = b[s], b[s + 1]
+            sl = int(state_slots[s])
+            if sl < 0 or r1 <= r0:
+                continue
+            S = state[sl].transpose(1, 2).clone() if int(positions[r0]) > 0 else \
+                torch.zeros((H, dk, dv), dtype=torch.float32)
+            for t in range(r0, r1):
+                S = decay[:, None, None] * S + kf[t][:, :, None] * vf[t][:, None, :]
+                out[t] = torch.einsum("hi,hij->hj", qf[t], S)
+            state[sl] = S.transpose(1, 2)
+        return out.view(T, H * dv)
+    out = torch.empty((T, n_heads * dv), dtype=torch.float32, device=q.device)
+    _m().retention(out.data_ptr(), state.data_ptr(), state.shape[0], q.data_ptr(), q.stride(0), k.data_ptr(),
+                   k.stride(0), v.data_ptr(), v.stride(0), decay.data_ptr(), float(k_scale), positions.data_ptr(),
+                   _ptr(seq_rows), state_slots.data_ptr(), n_seq, T, n_heads, dk, dv, _f32(q), _stream())
+    return out
+
+
+GATE_ACTS = {"sigmoid": 0, "silu": 1}
+
+
 def head_norm_gate(o: torch.Tensor, n_heads: int, weight: torch.Tensor | None, gate: torch.Tensor | None, eps: float,
-                   out_dtype: torch.dtype) -> torch.Tensor:
+                   out_dtype: torch.dtype, gate_act: str = "sigmoid") -> torch.Tensor:
     """o [T, H dv] fp32 -> every head divided by its root mean square
-    (sqrt(mean(o_h^2) + eps)), times weight [H dv] (fp32), times sigmoid(gate)
-    (gate [T, H dv], a column section of the activation dtype), in out_dtype."""
+    (sqrt(mean(o_h^2) + eps)), times weight [H dv] (fp32), times act(gate)
+    (gate [T, H dv], a column section of the activation dtype; gate_act
+    'sigmoid', or 'silu': z sigmoid(z)), in out_dtype."""
+    if gate_act not in GATE_ACTS:
+        raise ValueError(f"unknown gate activation {gate_act!r}")
     T, W = o.shape
     if o.dtype != torch.float32 or not o.is_contiguous() or W % n_heads:
         raise TypeError("head_norm_gate: o is contiguous float32 [T, H dv]")
@@ -241,9 +369,11 @@ def head_norm_gate(o: torch.Tensor, n_heads: int, weight: torch.Tensor | None, g
         if weight is not None:
             y = y * weight
         if gate is not None:
-            y = y * torch.sigmoid(gate.float())
+            g = gate.float()
+            y = y * (torch.sigmoid(g) if gate_act == "sigmoid" else g * torch.sigmoid(g))
         return y.to(out_dtype)
     out = torch.empty((T, W), dtype=out_dtype, device=o.device)
     _m().head_norm_gate(out.data_ptr(), o.data_ptr(), _ptr(weight), _ptr(gate), gate.stride(0) if gate is not None else 0,
-                        T, n_heads, W // n_heads, float(eps), int(out_dtype == torch.float32), _stream())
+                        T, n_heads, W // n_heads, float(eps), GATE_ACTS[gate_act], int(out_dtype == torch.float32),
+                        _stream())
     return out
