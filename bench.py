@@ -147,9 +147,9 @@ def parse(argv=None):
                          "measures the decode role of an xPyD layout whose decode engines prefill the other "
                          "1 - q of the prompts locally (1 = pure decode role)")
     ap.add_argument("--layered", action="store_true",
-                    help="instead of the headline workload: the layer-listed model families (Bekulix, Bolinex, Nefivik) beside Llama at "
+                    help="instead of the headline workload: the layer-listed model families (Bekulix, Bolinex, Nefivik, Sobivik) beside Llama at "
                          "equal layer sizes, prefill / decode tokens/s and attention kernels alone (one GPU)")
-    ap.add_argument("--layered-family", default="all", choices=["all", "bekulix", "bolinex", "nefivik"],
+    ap.add_argument("--layered-family", default="all", choices=["all", "bekulix", "bolinex", "nefivik", "sobivik"],
                     help="with --layered: which layer-listed family runs beside Llama")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--gemm-report", default=None, help="write the decode-GEMM tuning table (JSON) here")

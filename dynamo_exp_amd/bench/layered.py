@@ -1,6 +1,6 @@
-"""`bench.py --layered`: the layer-listed models (Bekulix, Bolinex, Nefivik) beside
-the closest existing model (Llama; for Nefivik also Bolinex, the closest
-layer-listed one) at equal layer sizes, random weights.
+"""`bench.py --layered`: the layer-listed models (Bekulix, Bolinex, Nefivik, Sobivik)
+beside the closest existing model (Llama; for Nefivik also Bolinex, for Sobivik
+also Bekulix, the closest layer-listed ones) at equal layer sizes, random weights.
 `--layered-family` picks which family runs (default: Bekulix and Bolinex).
 
 Two parts, both on one GPU:
@@ -24,7 +24,7 @@ import torch
 from .. import ops
 from ..engine.engine import EngineConfig, LLMEngine
 from ..engine.request import SamplingParams
-from ..models.config import ModelConfig, _bekulix_preset, _bolinex_preset, _nefivik_preset
+from ..models.config import ModelConfig, _bekulix_preset, _bolinex_preset, _nefivik_preset, _sobivik_preset
 from ..ops import mixers as mx
 from ..ops import moe
 from ..ops import recurrent as rc
@@ -60,6 +60,15 @@ def _nefivik_config(s: dict):
     of the dense width (two of four groups kept); token input of 256 columns."""
     return _nefivik_preset(f"nefivik {s['W']}", s["W"], s["layers"], s["H"], s["G"], s["d"], 1024, experts=8, top=2,
                            expert_ff=s["ff"] // 4, groups=(4, 2), side=256, vocab=s["vocab"], conv=4, attn_every=4)
+
+
+def _sobivik_config(s: dict):
+    """Sobivik at the size's layer shapes: differential attention (window 1024 that keeps the
+    first 64 tokens; half the heads at twice the value width), retention and latent attention
+    (rank 192 + 64 rotated columns, window 1024, sink) in turn, 4-tap input convolutions, dense
+    feed-forwards, the depth average after every layer."""
+    return _sobivik_preset(f"sobivik {s['W']}", s["W"], s["ff"], s["layers"], s["H"], s["G"], s["d"], 192,
+                           s["W"] // 4, 64, 1024, 64, vocab=s["vocab"])
 
 
 def _timed(fn, iters=10, warm=2) -> float:
@@ -420,6 +429,135 @@ def nefivik_kernels(s: dict, L: int, B: int, T: int) -> dict:
     return res
 
 
+def sobivik_kernels(s: dict, L: int, B: int, T: int) -> dict:
+    """Sobivik's kernels alone, each beside its counterpart: the retention scan beside the
+    delta-rule scan (4 prompts of L / 2 tokens; B decode rows); window attention with kept first
+    keys (two maps) and with a sink over one shared latent head, beside the same kernels without
+    either; the depth average (with the closing addend and the next norm) beside the residual
+    step; the input convolution and the latent / rotary preparation beside Nefivik's convolution +
+    rotation + cache write; the per-head norm with a silu gate beside the sigmoid one."""
+    H, G, d, W, bs = s["H"], s["G"], s["d"], s["W"], 64
+    dev, dt, win, keep = "cuda", torch.bfloat16, 1024, 64
+    res = {}
+
+    def put(name, us, byts=None, flops=None, **kw):
+        res[name] = {"us": round(us, 1), **kw}
+        if byts:
+            res[name]["TB/s"] = round(byts / us / 1e6, 2)
+        if flops:
+            res[name]["TFLOPs"] = round(flops / us / 1e6, 1)
+
+    # ---- the two scans: prompts, then decode rows
+    n = H * d
+    for tag, n_seq, rows in (("prefill", 4, L // 2), ("decode", B, 1)):
+        Tn = n_seq * rows
+        p = torch.randn(Tn, 5 * n, device=dev, dtype=dt)
+        state = torch.zeros(n_seq, H, d, d, device=dev)
+        pos = (torch.arange(rows, device=dev) + 1).repeat(n_seq)
+        seq_rows = torch.arange(0, Tn + 1, rows, dtype=torch.int32, device=dev) if rows > 1 else None
+        slots = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        decay = torch.full((H,), 0.97, device=dev)
+        st = n_seq * H * d * d * 4 * 2  # state read and written
+        us = _timed(lambda: rc.retention(p[:, :n], p[:, n:2 * n], p[:, 2 * n:3 * n], decay, d ** -0.5, state, pos,
+                                         seq_rows, slots, H, d, d))
+        put(f"retention_{tag}", us, Tn * n * (3 * 2 + 4) + st, 2.0 * 2 * Tn * H * d * d, tok_per_s=round(Tn / us * 1e6),
+            state_TBs=round(st / us / 1e6, 2))
+        wl = torch.randn(Tn, n, device=dev, dtype=dt)
+        zb = torch.zeros(n, device=dev)
+        us = _timed(lambda: rc.delta_rule(p[:, :n], p[:, n:2 * n], p[:, 2 * n:3 * n], p[:, 3 * n:4 * n], wl, zb, zb, state,
+                                          pos, seq_rows, slots, H, d, d))
+        put(f"nefivik_delta_rule_{tag}", us, Tn * n * (5 * 2 + 4) + st, 2.0 * 4 * Tn * H * d * d,
+            tok_per_s=round(Tn / us * 1e6), state_TBs=round(st / us / 1e6, 2))
+        o = torch.randn(Tn, n, device=dev)
+        for act in ("silu", "sigmoid"):
+            put(f"head_norm_gate_{act}_{tag}",
+                _timed(lambda: rc.head_norm_gate(o, H, None, p[:, 4 * n:5 * n], 1e-5, dt, gate_act=act)), Tn * n * (4 + 2 + 2))
+    # ---- attention: (name, query vectors, maps, group, d, dv, shared K/V row, extras)
+    Hd, Gd = H // 2, max(1, G // 2)
+    shapes = [("diff", 2 * Hd, 2, Hd // Gd, d, 2 * d, False, dict(keep_first=keep)),
+              ("latent", H, 1, H, 256, 192, True, dict(sink=torch.randn(H, device=dev)))]
+    nb = L // bs + 1
+    pos = torch.arange(L, device=dev)
+    seq = torch.zeros(L, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
+    tiles = torch.tensor(mx.tile_list(0, L), dtype=torch.int32, device=dev)
+    j = torch.arange(L)
+    vis = (j - mx.first_visible(j, "window", win) + 1)
+    nbb = B * nb
+    btd = torch.randperm(nbb, device=dev).to(torch.int32).view(B, nb)
+    posd = torch.full((B,), L - 1, device=dev)
+    for name, n_qh, maps, group, dd, dv, shared, extra in shapes:
+        n_kh, n_vh = n_qh // group, n_qh // maps // group
+        q = torch.randn(L, n_qh * dd, device=dev, dtype=dt)
+        kc = torch.randn(nb * bs, n_kh * dd, device=dev, dtype=dt)
+        vc = kc if shared else torch.randn(nb * bs, n_vh * dv, device=dev, dtype=dt)
+        sc = dd ** -0.5
+        for tag, kw in (("plain", {}), ("keep" if "keep_first" in extra else "sink", extra)):
+            seen = vis + (torch.minimum(torch.tensor(keep), mx.first_visible(j, "window", win)) if "keep_first" in kw else 0)
+            fl = 2.0 * (dd + dv) * n_qh * float(seen.sum())
+            us = _timed(lambda: mx.attention(q, kc, vc, pos, seq, bt, bs, n_qh, maps, group, dd, dv, sc, "window", win, 1,
+                                             maps == 2, tiles, L, **kw))
+            put(f"{name}_prefill_window{win}_{tag}", us, None, fl)
+        kcd = torch.randn(nbb * bs, n_kh * dd, device=dev, dtype=dt)
+        vcd = kcd if shared else torch.randn(nbb * bs, n_vh * dv, device=dev, dtype=dt)
+        qd = torch.randn(B, n_qh * dd, device=dev, dtype=dt)
+        parts = mx.row_attention_parts(B, n_kh * (-(-group // 32)), win, mx.GROUP_TARGET_WAVES)
+        for tag, kw in (("plain", {}), ("keep" if "keep_first" in extra else "sink", extra)):
+            rows_read = min(L, win) + (keep if "keep_first" in kw else 0)
+            byts = B * rows_read * (n_kh * dd + (0 if shared else n_vh * dv)) * 2
+            us = _timed(lambda: mx.attention(qd, kcd, vcd, posd, None, btd, bs, n_qh, maps, group, dd, dv, sc, "window",
+                                             win, parts, maps == 2, **kw))
+            put(f"{name}_decode_window{win}_{tag}", us, byts, parts=parts)
+    # ---- depth average (5 planes, closing addend, next norm) beside the residual step (addend, next norm)
+    planes = 5
+    stack = torch.randn(planes + 1, T, W, device=dev)
+    wts = torch.full((planes,), 1.0 / planes, device=dev)
+    c = torch.randn(T, W, device=dev, dtype=dt)
+    nw = torch.ones(W, device=dev)
+    put(f"depth_mix_{planes}_planes_addend_rmsnorm",
+        _timed(lambda: mx.depth_mix(stack, planes, wts, dst=stack[planes], norm_w=nw, eps=1e-5, out_dtype=dt, c=c, c_w=nw)),
+        T * W * (4 * planes + 4 + 4 + 2 + 2 + 2))  # planes read, newest written back, sum written, addend (twice), norm out
+    X = torch.randn(T, W, device=dev)
+    put("residual_step_unit_rms_addend_rmsnorm",
+        _timed(lambda: mx.residual_step(X, c=c, c_w=nw, eps=1e-5, norm="rms", norm_w=nw, out_dtype=dt)),
+        T * W * (4 + 4 + 2 + 2))
+    # ---- input convolution (all W channels) and latent / rotary preparation beside Nefivik's convolution + rotation
+    taps = 4
+    x = torch.randn(T, W, device=dev, dtype=dt)
+    cw = torch.randn(taps, W, device=dev)
+    tail = torch.zeros(1, taps - 1, W, device=dev, dtype=dt)
+    posT = torch.arange(T, device=dev)
+    rs = torch.zeros(T, dtype=torch.int32, device=dev)
+    sr = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    s0 = torch.zeros(1, dtype=torch.int32, device=dev)
+    put("input_conv", _timed(lambda: rc.conv_rope_cache(x, cw, tail, posT, posT, rs, sr, s0, 1, 0, W, 0, None, None, None)),
+        T * W * 2 * 2)
+    C = (H + 2 * G) * d
+    xq = torch.randn(T, C, device=dev, dtype=dt)
+    cwq = torch.randn(taps, C, device=dev)
+    tailq = torch.zeros(1, taps - 1, C, device=dev, dtype=dt)
+    nbt = T // bs + 1
+    kcn = torch.zeros(nbt * bs, G * d, device=dev, dtype=dt)
+    vcn = torch.zeros_like(kcn)
+    inv = rc.rotary_frequencies(d // 2, 500000.0, None).to(dev)
+    put("nefivik_conv_rope_cache",
+        _timed(lambda: rc.conv_rope_cache(xq, cwq, tailq, posT, posT, rs, sr, s0, H, G, d, d, inv, kcn, vcn)),
+        T * d * 2 * (2 * H + 4 * G))
+    r, dr = 192, 64
+    qa = torch.randn(H, T, r, device=dev, dtype=dt)
+    qp = torch.randn(T, H * (d + dr), device=dev, dtype=dt)
+    kv = torch.randn(T, r + dr, device=dev, dtype=dt)
+    cn = torch.ones(r, device=dev)
+    fr, mag = rc.yarn_frequencies(dr, 10000.0, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+    cache = torch.zeros(nbt * bs, r + dr, device=dev, dtype=dt)
+    put("latent_rope", _timed(lambda: rc.latent_rope(qa, qp, d + dr, d, kv, r, dr, cn, 1e-5, fr.to(dev), mag, posT, posT,
+                                                      cache)), T * 2 * (2 * H * (r + dr) + 2 * (r + dr)))
+    sn = torch.randn(T, W // 4 + r + dr, device=dev, dtype=dt)
+    qn = torch.ones(W // 4, device=dev)
+    put("section_norm", _timed(lambda: mx.section_norm(sn[:, :W // 4], qn, 1e-5)), T * (W // 4) * 2 * 2)
+    return res
+
+
 def run_layered_compare(args, dev) -> dict:
     isl, osl = min(args.isl, 2048), min(args.osl, 64)
     fam = getattr(args, "layered_family", "all")
@@ -432,18 +570,22 @@ def run_layered_compare(args, dev) -> dict:
         if fam in ("all", "bolinex"):
             row["bolinex"] = engine_throughput(_bolinex_config(s), dev, isl, osl, 4, 64, args.seed)
             row["bolinex_kernels"] = bolinex_kernels(s, 4096, 64, 8192)
+        if fam == "sobivik":
+            row["sobivik"] = engine_throughput(_sobivik_config(s), dev, isl, osl, 4, 64, args.seed)
+            row["sobivik_kernels"] = sobivik_kernels(s, 4096, 64, 8192)
+            row["bekulix"] = engine_throughput(bek, dev, isl, osl, 4, 64, args.seed)
         if fam == "nefivik":
             row["nefivik"] = engine_throughput(_nefivik_config(s), dev, isl, osl, 4, 64, args.seed)
             row["nefivik_kernels"] = nefivik_kernels(s, 4096, 64, 8192)
             row["bolinex"] = engine_throughput(_bolinex_config(s), dev, isl, osl, 4, 64, args.seed)
         row["llama"] = engine_throughput(lla, dev, isl, osl, 4, 64, args.seed)
-        if fam == "nefivik":
+        if fam in ("nefivik", "sobivik"):
             sizes[name] = row
             continue
         row["attention_kernels"] = attention_kernels(s, 4096, 64)
         if fam in ("all", "bekulix"):
             row["rowwise_kernels"] = rowwise_kernels(s, 8192)
         sizes[name] = row
-    return {"metric": "layer-listed models (Bekulix, Bolinex, Nefivik) beside Llama at equal layer sizes: engine prefill / "
+    return {"metric": "layer-listed models (Bekulix, Bolinex, Nefivik, Sobivik) beside Llama at equal layer sizes: engine prefill / "
                       "decode tokens/s and kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
             "family": fam, "data": "synthetic (random-token prompts, random-init weights)", "sizes": sizes}

@@ -19,8 +19,8 @@ int dxm_stream_step(float*, const void*, int64_t, const float*, const float*, co
 int dxm_embed_streams(float*, const void*, const int64_t*, int, int, int, int64_t, const void*, const int64_t*,
                       int64_t, float, int, hipStream_t);
 int dxm_section_norm(void*, const void*, int64_t, const float*, int, int, float, int, hipStream_t);
-int dxm_depth_mix(float*, const float*, int64_t, int, const float*, const int64_t*, int, float, const float*, void*, int,
-                  int, hipStream_t);
+int dxm_depth_mix(float*, float*, int64_t, int, const float*, const int64_t*, int, float, const float*, void*,
+                  const void*, int64_t, const float*, int, int, hipStream_t);
 int dxm_retention(float*, float*, int, const void*, int64_t, const void*, int64_t, const void*, int64_t, const float*,
                   float, const int64_t*, const int*, const int*, int, int, int, int, int, int, hipStream_t);
 int dxm_latent_rope(void*, const void*, const void*, int64_t, int, int, const void*, int64_t, const float*, float,
@@ -92,10 +92,10 @@ PYBIND11_MODULE(_C_mixers, m) {
   m.def("section_norm", [](u out, u x, int64_t xs, u w, int rows, int n, float eps, int f32, u st) {
     check(dxm_section_norm(P(out), P(x), xs, F(w), rows, n, eps, f32, S(st)), "section_norm");
   });
-  m.def("depth_mix", [](u dst, u stack, int64_t plane, int n, u w, u rows, int n_rows, float eps, u nw, u out, int W,
-                        int f32, u st) {
+  m.def("depth_mix", [](u dst, u stack, int64_t plane, int n, u w, u rows, int n_rows, float eps, u nw, u out, u c,
+                        int64_t cs, u cw, int W, int f32, u st) {
     check(dxm_depth_mix(F(dst), F(stack), plane, n, F(w), reinterpret_cast<const int64_t*>(rows), n_rows, eps, F(nw),
-                        P(out), W, f32, S(st)),
+                        P(out), P(c), cs, F(cw), W, f32, S(st)),
           "depth_mix");
   });
   m.def("retention", [](u out, u state, int n_slots, u q, int64_t qs, u k, int64_t ks, u v, int64_t vs, u decay,

@@ -339,33 +339,62 @@ __global__ void __launch_bounds__(kThreads) residual_step_kernel(
 //     dst[r, :] = sum_{j < n} w[j] * stack[j][row(r), :]        row(r) = rows ? rows[r] : r
 // stack [>= n, T, W] fp32, one [T, W] plane per layer result; dst fp32 [n_rows, W] (it may be a
 // later plane of the same stack); then, when out: out = dst / sqrt(mean(dst^2) + eps) * nw in T
-// (nw one weight per column).  Sums in the order j = 0, 1, ..., all fp32.  The row stays in
-// registers between the sum and the norm (W <= kThreads * V * kResChunks) or is re-read from dst.
+// (nw one weight per column).  With c (the last sublayer's output, [T, c_stride] in T) the newest
+// plane n - 1 first takes its closing addend, plane <- plane + c / sqrt(mean(c^2) + eps) * cw, and
+// is written back (without `rows`; with them the sum alone uses it, a row may be listed twice).
+// Sums in the order j = 0, 1, ..., all fp32.  The row stays in registers between the sum and the
+// norm (W <= kThreads * V * kResChunks) or is re-read from dst.
 template <typename T, int V>
-__global__ void __launch_bounds__(kThreads) depth_mix_kernel(float* __restrict__ dst, const float* __restrict__ stack,
+__global__ void __launch_bounds__(kThreads) depth_mix_kernel(float* __restrict__ dst, float* __restrict__ stack,
                                                              int64_t plane, int n, const float* __restrict__ w,
                                                              const int64_t* __restrict__ rows, float eps,
-                                                             const float* __restrict__ nw, T* __restrict__ out, int W) {
+                                                             const float* __restrict__ nw, T* __restrict__ out,
+                                                             const T* __restrict__ c, int64_t c_stride,
+                                                             const float* __restrict__ cw, int W) {
   __shared__ float red[16];
   const int64_t r = blockIdx.x;
   const int64_t row = rows ? rows[r] : r;
-  const float* src = stack + row * (int64_t)W;
+  float* src = stack + row * (int64_t)W;
   float* x = dst + r * (int64_t)W;
+  float rc = 0.f;
+  if (c) {
+    float cs = 0.f;
+    for (int e = threadIdx.x * V; e < W; e += kThreads * V) {
+      float t[V];
+      ldv<T, V>(c + row * c_stride + e, t);
+#pragma unroll
+      for (int i = 0; i < V; ++i) cs += t[i] * t[i];
+    }
+    rc = rsqrtf(block_reduce_sum(cs, red) / (float)W + eps);
+    __syncthreads();
+  }
+  // the weighted sum of columns e .. e + V - 1 over the planes
+  auto mix = [&](int e, float* a) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) a[i] = 0.f;
+    for (int j = 0; j < n; ++j) {
+      float t[V];
+      ldv<float, V>(src + j * plane + e, t);
+      if (c && j == n - 1) {
+        float cv[V], g[V];
+        ldv<T, V>(c + row * c_stride + e, cv);
+        ldv<float, V>(cw + e, g);
+#pragma unroll
+        for (int i = 0; i < V; ++i) t[i] += cv[i] * rc * g[i];
+        if (!rows) stv<float, V>(src + j * plane + e, t);
+      }
+      const float wj = w[j];
+#pragma unroll
+      for (int i = 0; i < V; ++i) a[i] += wj * t[i];
+    }
+  };
   float acc[kResChunks][V];
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < kResChunks; ++k) {
     const int e = (threadIdx.x + k * kThreads) * V;
     if (e < W) {
-#pragma unroll
-      for (int i = 0; i < V; ++i) acc[k][i] = 0.f;
-      for (int j = 0; j < n; ++j) {
-        float t[V];
-        ldv<float, V>(src + j * plane + e, t);
-        const float wj = w[j];
-#pragma unroll
-        for (int i = 0; i < V; ++i) acc[k][i] += wj * t[i];
-      }
+      mix(e, acc[k]);
       stv<float, V>(x + e, acc[k]);
 #pragma unroll
       for (int i = 0; i < V; ++i) ss += acc[k][i] * acc[k][i];
@@ -373,15 +402,7 @@ __global__ void __launch_bounds__(kThreads) depth_mix_kernel(float* __restrict__
   }
   for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
     float a[V];
-#pragma unroll
-    for (int i = 0; i < V; ++i) a[i] = 0.f;
-    for (int j = 0; j < n; ++j) {
-      float t[V];
-      ldv<float, V>(src + j * plane + e, t);
-      const float wj = w[j];
-#pragma unroll
-      for (int i = 0; i < V; ++i) a[i] += wj * t[i];
-    }
+    mix(e, a);
     stv<float, V>(x + e, a);
 #pragma unroll
     for (int i = 0; i < V; ++i) ss += a[i] * a[i];
@@ -714,19 +735,21 @@ int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int6
   return 0;
 }
 
-int dxm_depth_mix(float* dst, const float* stack, int64_t plane, int n, const float* w, const int64_t* rows, int n_rows,
-                  float eps, const float* nw, void* out, int W, int f32, hipStream_t st) {
+int dxm_depth_mix(float* dst, float* stack, int64_t plane, int n, const float* w, const int64_t* rows, int n_rows,
+                  float eps, const float* nw, void* out, const void* c, int64_t c_stride, const float* cw, int W,
+                  int f32, hipStream_t st) {
   if (n_rows <= 0) return 0;
-  if (n < 1 || W < 1 || !dst || !stack || !w || (out && !nw)) return 1;
+  if (n < 1 || W < 1 || !dst || !stack || !w || (out && !nw) || (c && !cw)) return 1;
   const int esz = f32 ? 4 : 2;
   auto al = [&](const void* p, int by) { return (uintptr_t)p % by == 0; };
-  const bool vec = W % 4 == 0 && plane % 4 == 0 && al(dst, 16) && al(stack, 16) && al(nw, 16) && al(out, 4 * esz);
+  const bool vec = W % 4 == 0 && plane % 4 == 0 && c_stride % 4 == 0 && al(dst, 16) && al(stack, 16) && al(nw, 16) &&
+                   al(out, 4 * esz) && al(c, 4 * esz) && al(cw, 16);
   if (vec) {
     DISPATCH_T(f32, hipLaunchKernelGGL((depth_mix_kernel<T, 4>), dim3(n_rows), dim3(kThreads), 0, st, dst, stack, plane,
-                                       n, w, rows, eps, nw, (T*)out, W));
+                                       n, w, rows, eps, nw, (T*)out, (const T*)c, c_stride, cw, W));
   } else {
     DISPATCH_T(f32, hipLaunchKernelGGL((depth_mix_kernel<T, 1>), dim3(n_rows), dim3(kThreads), 0, st, dst, stack, plane,
-                                       n, w, rows, eps, nw, (T*)out, W));
+                                       n, w, rows, eps, nw, (T*)out, (const T*)c, c_stride, cw, W));
   }
   DX_CHECK_LAUNCH();
   return 0;

@@ -33,7 +33,9 @@ average of planes 0 .. i) and is updated in place into layer i's result:
     ym = (a @ Wuv (per head) * sigmoid(p_g)) @ Wo^T        batched GEMM + HIP act_mul
   all
     x += rms(ym) g1b; h2 = rms(x) g2                       HIP  residual_step
-    x += rms(ff(h2)) g2b                                   hipBLASLt + HIP glu_act (silu) + residual_step
+    yf = ff(h2)                                            hipBLASLt + HIP glu_act (silu)
+    x += rms(yf) g2b                                       joined with the next layer's depth_mix (or the final one,
+                                                           on the chosen rows)
 
 Norms, the residual and its depth average, scores and weights, decays and the
 retention state, positions and angles are fp32; projections, the convolution
@@ -456,21 +458,22 @@ class SobivikForCausalLM:
                 self.layer_hook(i)
             if L["mlp"]:
                 h2, _ = mx.residual_step(X, c=y, c_w=L["norm1b"], norm="rms", norm_w=L["norm2"], **rs)
-                f = self._mm(mx.glu_act(self._mm(h2, L["w_gu"]), "silu"), L["w_down"])
-                mx.residual_step(X, c=f, c_w=L["norm2b"], **rs)
+                pend = dict(c=self._mm(mx.glu_act(self._mm(h2, L["w_gu"]), "silu"), L["w_down"]), c_w=L["norm2b"])
             else:
-                mx.residual_step(X, c=y, c_w=L["norm1b"], **rs)
-            # X (plane i + 1) is the layer's result; what goes on is the average over planes 0 .. i + 1
+                pend = dict(c=y, c_w=L["norm1b"])
+            # the addend that closes the layer joins plane i + 1, the layer's result, in the pass that
+            # forms what goes on: the average over planes 0 .. i + 1 (and the next layer's norm)
+            if self.trace_layers is not None:
+                mx.residual_step(X, **pend, **rs)
+                pend = {}
+                self.trace_layers.append(mx.depth_mix(stack, i + 2, L["dwa"])[0])
             if i + 1 < n:
-                X, h = mx.depth_mix(stack, i + 2, L["dwa"], dst=stack[i + 2], norm_w=self.layers[i + 1]["norm1"], **rs)
-                if self.trace_layers is not None:
-                    self.trace_layers.append(X.clone())
-        if self.trace_layers is not None:
-            self.trace_layers.append(mx.depth_mix(stack, n + 1, self.layers[-1]["dwa"])[0])
+                X, h = mx.depth_mix(stack, i + 2, L["dwa"], dst=stack[i + 2], norm_w=self.layers[i + 1]["norm1"],
+                                    **pend, **rs)
         if pick is not None and pick.numel() == 0:
             return torch.empty((0, W), device=stack.device, dtype=dt)
         # the last average and the final norm, on the chosen rows only
-        return mx.depth_mix(stack, n + 1, self.layers[-1]["dwa"], rows=pick, norm_w=self.final_w, **rs)[1]
+        return mx.depth_mix(stack, n + 1, self.layers[-1]["dwa"], rows=pick, norm_w=self.final_w, **pend, **rs)[1]
 
     def compute_logits(self, hidden: torch.Tensor, fp32: bool = False) -> torch.Tensor:
         """Logits of final-normed rows, times the model's logit scale; fp32:

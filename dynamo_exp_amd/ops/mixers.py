@@ -217,7 +217,8 @@ def section_norm(x: torch.Tensor, weight: torch.Tensor | None, eps: float) -> to
 
 def depth_mix(stack: torch.Tensor, n: int, weights: torch.Tensor, dst: torch.Tensor | None = None,
               rows: torch.Tensor | None = None, norm_w: torch.Tensor | None = None, eps: float = 1e-6,
-              out_dtype: torch.dtype = torch.bfloat16):
+              out_dtype: torch.dtype = torch.bfloat16, c: torch.Tensor | None = None,
+              c_w: torch.Tensor | None = None):
     """A weighted sum over depth: stack [>= n, T, W] fp32 holds one [T, W]
     plane per layer result (plane 0 the embedding output);
         x[r] = sum_{j < n} weights[j] * stack[j, rows[r]]        (rows None: every row)
@@ -225,24 +226,37 @@ def depth_mix(stack: torch.Tensor, n: int, weights: torch.Tensor, dst: torch.Ten
     [len(rows) or T, W]; a later plane of the stack is the usual choice, so the
     next layer updates it in place into its own result) and returned together
     with norm(x) = x / sqrt(mean(x^2) + eps) * norm_w in out_dtype (None without
-    norm_w)."""
+    norm_w).  With c [T, W] (the last sublayer's output, of out_dtype) the newest
+    plane first takes its closing addend, stack[n - 1] += c / sqrt(mean(c^2) +
+    eps) * c_w: the residual step that ends a layer, in the same pass.  With
+    `rows` the plane itself is left as it was (only the sum uses the addend)."""
     if stack.dim() != 3 or stack.dtype != torch.float32 or not stack.is_contiguous() or not 1 <= n <= stack.shape[0]:
         raise TypeError("depth_mix: stack is contiguous float32 [planes, T, W] with n <= planes")
     _, T, W = stack.shape
     _fp32_param(weights, "weights")
     _fp32_param(norm_w, "norm_w")
+    _fp32_param(c_w, "c_w")
     if weights.numel() != n or (norm_w is not None and norm_w.numel() != W):
         raise ValueError("depth_mix: one weight per plane, one norm weight per column")
+    if c is not None and (c_w is None or c_w.numel() != W or c.shape != (T, W) or c.stride(1) != 1 or
+                          c.dtype != out_dtype):
+        raise ValueError("depth_mix: the addend is [T, W] of the activation dtype with a weight per column")
     R = T if rows is None else rows.numel()
     if dst is None:
         dst = torch.empty((R, W), dtype=torch.float32, device=stack.device)
     if dst.shape != (R, W) or dst.dtype != torch.float32 or not dst.is_contiguous():
         raise TypeError("depth_mix: dst is contiguous float32 [rows, W]")
     if not stack.is_cuda:
-        src = stack[:n] if rows is None else stack[:n, rows.long()]
+        last = stack[n - 1]
+        if c is not None:
+            cf = c.float()
+            last = last + cf * torch.rsqrt((cf * cf).mean(-1, keepdim=True) + eps) * c_w
+            if rows is None:
+                stack[n - 1] = last
+        planes = [stack[j] for j in range(n - 1)] + [last]
         x = torch.zeros((R, W), dtype=torch.float32)
         for j in range(n):
-            x += weights[j] * src[j]
+            x += weights[j] * (planes[j] if rows is None else planes[j][rows.long()])
         dst.copy_(x)
         h = None
         if norm_w is not None:
@@ -252,7 +266,8 @@ def depth_mix(stack: torch.Tensor, n: int, weights: torch.Tensor, dst: torch.Ten
         raise TypeError("depth_mix: rows must be contiguous int64")
     h = torch.empty((R, W), dtype=out_dtype, device=stack.device) if norm_w is not None else None
     _m().depth_mix(dst.data_ptr(), stack.data_ptr(), T * W, n, weights.data_ptr(), _ptr(rows), R, float(eps),
-                   _ptr(norm_w), _ptr(h), W, int(out_dtype == torch.float32), _stream())
+                   _ptr(norm_w), _ptr(h), _ptr(c), c.stride(0) if c is not None else 0, _ptr(c_w), W,
+                   int(out_dtype == torch.float32), _stream())
     return dst, h
 
 

@@ -246,6 +246,18 @@ def test_depth_mix_alone(device, W, n):
     rows = torch.tensor([4, 0, 4], device=device)
     x, h = mx.depth_mix(sd, n, w.to(device), rows=rows)
     assert h is None and torch.allclose(x.cpu().double(), want[rows.cpu()], atol=2e-5)
+    # with the addend that closes the newest plane's layer: the plane is updated in the same pass
+    # (all rows), or left alone while the sum uses the addend (chosen rows, one listed twice)
+    c, cw = torch.randn(T, W + 4) * 3, torch.randn(W)
+    last = stack[n - 1].double() + O.unit_rms(c[:, 4:].double(), eps) * cw.double()
+    want = O.depth_average([stack[j].double() for j in range(n - 1)] + [last], w.double())
+    x, _ = mx.depth_mix(sd, n, w.to(device), rows=rows, eps=eps, out_dtype=torch.float32, c=c.to(device)[:, 4:],
+                        c_w=cw.to(device))
+    assert torch.allclose(x.cpu().double(), want[rows.cpu()], atol=3e-5) and torch.equal(sd[n - 1].cpu(), stack[n - 1])
+    x, h = mx.depth_mix(sd, n, w.to(device), dst=sd[n], norm_w=nw.to(device), eps=eps, out_dtype=torch.float32,
+                        c=c.to(device)[:, 4:], c_w=cw.to(device))
+    assert torch.allclose(sd[n - 1].cpu().double(), last, atol=2e-5) and torch.allclose(x.cpu().double(), want, atol=3e-5)
+    assert torch.allclose(h.cpu().double(), O.unit_rms(want, eps) * nw.double(), atol=5e-5)
 
 
 @pytest.mark.parametrize("device", DEVICES)
