@@ -44,7 +44,9 @@ struct LatentArgs {
   int T, H, r, dr;
 };
 
-template <typename T>
+// VEC: elements per 16-byte chunk when r, dr, the row strides and the bases allow whole chunks
+// (the query parts, the bulk of the bytes, are then copied chunk by chunk), else 1
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256) latent_rope_kernel(LatentArgs g) {
   extern __shared__ float cs_sn[];  // [half] cosines, [half] sines, both times mag
   __shared__ float red[16];
@@ -81,10 +83,26 @@ __global__ void __launch_bounds__(256) latent_rope_kernel(LatentArgs g) {
   }
   const T* q = (const T*)g.q + t * g.q_stride;
   T* qo = (T*)g.q_out + t * (int64_t)g.H * Wc;
-  for (int it = tid; it < g.H * Wc; it += blockDim.x) {
-    const int h = it / Wc, c = it - h * Wc;
-    if (c < g.r) qo[it] = ((const T*)g.qa)[((int64_t)h * g.T + t) * g.r + c];
-    else stf<T>(qo, it, rot(q + (int64_t)h * g.q_head + g.q_off, c - g.r));
+  if constexpr (VEC > 1) {
+    typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
+    const int per = Wc / VEC;
+    for (int it = tid; it < g.H * per; it += blockDim.x) {
+      const int h = it / per, c = (it - h * per) * VEC;
+      if (c < g.r) {
+        *reinterpret_cast<raw4*>(qo + (int64_t)h * Wc + c) =
+            *reinterpret_cast<const raw4*>((const T*)g.qa + ((int64_t)h * g.T + t) * g.r + c);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          stf<T>(qo, (int64_t)h * Wc + c + e, rot(q + (int64_t)h * g.q_head + g.q_off, c - g.r + e));
+      }
+    }
+  } else {
+    for (int it = tid; it < g.H * Wc; it += blockDim.x) {
+      const int h = it / Wc, c = it - h * Wc;
+      if (c < g.r) qo[it] = ((const T*)g.qa)[((int64_t)h * g.T + t) * g.r + c];
+      else stf<T>(qo, it, rot(q + (int64_t)h * g.q_head + g.q_off, c - g.r));
+    }
   }
 }
 
@@ -101,8 +119,12 @@ extern "C" int dxm_latent_rope(void* q_out, const void* qa, const void* q, int64
   LatentArgs g{q_out, qa, q, q_stride, q_head, q_off, kv, kv_stride, cn, eps, inv_freq, half, mag,
                pos, slots, cache, T_, H, r, dr};
   const size_t lds = (size_t)2 * half * sizeof(float);
-  if (f32) hipLaunchKernelGGL(latent_rope_kernel<float>, dim3(T_), dim3(256), lds, st, g);
-  else hipLaunchKernelGGL(latent_rope_kernel<bf16_t>, dim3(T_), dim3(256), lds, st, g);
+  const int V = f32 ? 4 : 8;
+  const bool vec = r % V == 0 && dr % V == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)qa % 16 == 0;
+  if (f32 && vec) hipLaunchKernelGGL((latent_rope_kernel<float, 4>), dim3(T_), dim3(256), lds, st, g);
+  else if (f32) hipLaunchKernelGGL((latent_rope_kernel<float, 1>), dim3(T_), dim3(256), lds, st, g);
+  else if (vec) hipLaunchKernelGGL((latent_rope_kernel<bf16_t, 8>), dim3(T_), dim3(256), lds, st, g);
+  else hipLaunchKernelGGL((latent_rope_kernel<bf16_t, 1>), dim3(T_), dim3(256), lds, st, g);
   DX_CHECK_LAUNCH();
   return 0;
 }

@@ -412,8 +412,144 @@ __global__ void __launch_bounds__(256) retention_kernel(RetArgs g) {
   }
 }
 
+// The same for key widths dk = 16 R and 16-byte aligned operands: nothing in the token loop is
+// conditional.  Lane r of a column's group owns the four row quads 4 (r + R qd) .. + 3, qd < 4, so
+// a group's 128-bit LDS reads of a q or k row are neighbouring chunks and the state is read and
+// written as 16-byte runs.  The next block's eight tokens (q, k of the head, v of the workgroup's
+// columns) are fetched into registers as 16-byte chunks while the current block's chain runs.
+typedef uint32_t ret_u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> __device__ __forceinline__ void chunk_to_f32(const ret_u32x4& c, float* o);
+template <> __device__ __forceinline__ void chunk_to_f32<bf16_t>(const ret_u32x4& c, float* o) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[2 * i] = bf16lo(c[i]), o[2 * i + 1] = bf16hi(c[i]);
+}
+template <> __device__ __forceinline__ void chunk_to_f32<float>(const ret_u32x4& c, float* o) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = __uint_as_float(c[i]);
+}
+
+template <typename T, int R>
+__global__ void __launch_bounds__(256) retention_fast_kernel(RetArgs g) {
+  constexpr int dk = 16 * R, cols = 256 / R, VEC = 16 / (int)sizeof(T);
+  constexpr int QC = dk / VEC, VC = cols / VEC;          // chunks per token row
+  constexpr int QK_CH = kTok * QC, V_CH = kTok * VC, N_CH = 2 * QK_CH + V_CH;
+  constexpr int PER = (N_CH + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs_[kTok * dk];
+  __shared__ __attribute__((aligned(16))) float ks_[kTok * dk];
+  __shared__ __attribute__((aligned(16))) float vs_[kTok * cols];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, cl = tid / R, r = tid % R;
+  const int col0 = blockIdx.z * cols, j = col0 + cl;
+  const int r0 = g.seq_rows ? g.seq_rows[s] : s, r1 = g.seq_rows ? g.seq_rows[s + 1] : s + 1;
+  if (r1 <= r0 || r0 < 0 || r1 > g.T) return;
+  const int slot = g.slots[s];
+  const int64_t ow = (int64_t)g.H * g.dv;
+  if (slot < 0 || slot >= g.n_slots) {  // a padding row: zeros out, no state touched
+    for (int t = r0; t < r1; ++t)
+      if (r == 0) g.out[(int64_t)t * ow + h * g.dv + j] = 0.f;
+    return;
+  }
+  float* sp = g.state + (((int64_t)slot * g.H + h) * g.dv + j) * dk;
+  const bool fresh = g.pos[r0] == 0;
+  float S[16];
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    const f32x4 v4 = fresh ? f32x4{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const f32x4*>(sp + 4 * (r + R * qd));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) S[4 * qd + e] = v4[e];
+  }
+  const float dec = g.decay[h];
+  const T* q = (const T*)g.q + (int64_t)h * dk;
+  const T* k = (const T*)g.k + (int64_t)h * dk;
+  const T* v = (const T*)g.v + (int64_t)h * g.dv + col0;
+  ret_u32x4 pf[PER];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = tid + i * 256;
+      const T* src = nullptr;
+      if (c < QK_CH) {
+        const int tt = c / QC;
+        if (t0 + tt < r1) src = q + (int64_t)(t0 + tt) * g.qs + (c % QC) * VEC;
+      } else if (c < 2 * QK_CH) {
+        const int c2 = c - QK_CH, tt = c2 / QC;
+        if (t0 + tt < r1) src = k + (int64_t)(t0 + tt) * g.ks + (c2 % QC) * VEC;
+      } else if (c < N_CH) {
+        const int c2 = c - 2 * QK_CH, tt = c2 / VC;
+        if (t0 + tt < r1) src = v + (int64_t)(t0 + tt) * g.vs + (c2 % VC) * VEC;
+      }
+      pf[i] = src ? *reinterpret_cast<const ret_u32x4*>(src) : ret_u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = tid + i * 256;
+      float f[VEC];
+      chunk_to_f32<T>(pf[i], f);
+      float* dst = nullptr;
+      if (c < QK_CH) {
+        dst = qs_ + c * VEC;
+      } else if (c < 2 * QK_CH) {
+        dst = ks_ + (c - QK_CH) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) f[e] *= g.k_scale;
+      } else if (c < N_CH) {
+        dst = vs_ + (c - 2 * QK_CH) * VEC;
+      }
+      if (dst) {
+#pragma unroll
+        for (int e = 0; e < VEC; e += 4) *reinterpret_cast<f32x4*>(dst + e) = f32x4{f[e], f[e + 1], f[e + 2], f[e + 3]};
+      }
+    }
+  };
+  fetch(r0);
+  for (int t0 = r0; t0 < r1; t0 += kTok) {
+    const int nt = r1 - t0 < kTok ? r1 - t0 : kTok;
+    __syncthreads();  // the previous block's reads are done
+    commit();
+    __syncthreads();
+    if (t0 + kTok < r1) fetch(t0 + kTok);
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vj = vs_[tt * cols + cl];
+      float acc = 0.f;
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const f32x4 kk = *reinterpret_cast<const f32x4*>(ks_ + tt * dk + 4 * (r + R * qd));
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(qs_ + tt * dk + 4 * (r + R * qd));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          S[4 * qd + e] = dec * S[4 * qd + e] + kk[e] * vj;
+          acc += qq[e] * S[4 * qd + e];
+        }
+      }
+      acc = group_sum<R>(acc);
+      if (r == 0) g.out[(int64_t)(t0 + tt) * ow + h * g.dv + j] = acc;
+    }
+  }
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd)
+    *reinterpret_cast<f32x4*>(sp + 4 * (r + R * qd)) = f32x4{S[4 * qd], S[4 * qd + 1], S[4 * qd + 2], S[4 * qd + 3]};
+}
+
+// whether the unconditional kernel serves the launch: dk = 16 R exactly, whole column blocks,
+// 16-byte aligned rows and sections
+template <typename T, int R>
+bool retention_fast_ok(const RetArgs& g) {
+  constexpr int VEC = 16 / (int)sizeof(T), cols = 256 / R;
+  auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
+  return g.dk == 16 * R && g.dv % cols == 0 && cols % VEC == 0 && g.qs % VEC == 0 && g.ks % VEC == 0 &&
+         g.vs % VEC == 0 && al(g.q) && al(g.k) && al(g.v) && al(g.state);
+}
+
 template <typename T, int R>
 void launch_retention(const RetArgs& g, int n_seq, hipStream_t st) {
+  if (retention_fast_ok<T, R>(g)) {
+    hipLaunchKernelGGL((retention_fast_kernel<T, R>), dim3(n_seq, g.H, g.dv / (256 / R)), dim3(256), 0, st, g);
+    return;
+  }
+
   int nt = (R * g.dv + 63) / 64 * 64;
   nt = nt > 256 ? 256 : nt;
   const int cols = nt / R;

@@ -160,16 +160,18 @@ def paged(T, bs, n_blocks, width, device, dtype, seed=3):
 
 
 # ----------------------------------------------------------------- mechanisms alone
-@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("H,dk,dv", [(2, 16, 16), (3, 10, 14), (1, 64, 64), (2, 128, 40), (1, 34, 3), (1, 200, 70),
-                                     (1, 1, 1)])
-def test_retention_alone(device, H, dk, dv):
+                                     (1, 1, 1), (2, 128, 64), (1, 32, 256), (2, 256, 32), (1, 16, 256)])
+def test_retention_alone(device, dtype, H, dk, dv):
     """Two sequences scanned whole, then in steps of unequal portions (19, 2, 1, ...) in slots that hold
-    garbage, then a decode step with a padding row, against the token-by-token oracle."""
+    garbage, then a decode step with a padding row, against the token-by-token oracle (over the
+    bf16 values of the inputs where those are bf16; the scan itself is fp32 either way)."""
     torch.manual_seed(dk)
     T = 41
-    q, k = torch.randn(2, T, H * dk), torch.randn(2, T, H * dk)
-    v = torch.randn(2, T, H * dv)
+    dt = DT[dtype]
+    q, k = torch.randn(2, T, H * dk).to(dt), torch.randn(2, T, H * dk).to(dt)
+    v = torch.randn(2, T, H * dv).to(dt)
     decay = torch.tensor([1.0 - 2.0 ** -(1 + h) for h in range(H)])
     ks = dk ** -0.5
     want = [O.retention_scan(q[s].double().view(T, H, dk), k[s].double().view(T, H, dk) * ks,
@@ -195,9 +197,9 @@ def test_retention_alone(device, H, dk, dv):
                                   rtol=1e-4)
     pos = torch.tensor([T, T, 0], device=device)
     slots = torch.tensor([3, 1, -1], dtype=torch.int32, device=device)
-    x = torch.randn(3, H * dk)
+    x = torch.randn(3, H * dk).to(dt)
     before = state[[0, 2, 4]].clone()
-    o = rc.retention(d(x), d(x), d(torch.randn(3, H * dv)), d(decay), ks, state, pos, None, slots, H, dk, dv)
+    o = rc.retention(d(x), d(x), d(torch.randn(3, H * dv).to(dt)), d(decay), ks, state, pos, None, slots, H, dk, dv)
     assert bool(torch.isfinite(o).all()) and float(o[2].abs().max()) == 0.0
     assert torch.equal(state[[0, 2, 4]], before)  # other slots are not touched
 
