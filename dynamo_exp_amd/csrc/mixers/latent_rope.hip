@@ -25,6 +25,35 @@ template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float
 template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
 
+// VEC consecutive elements as floats, one 16-byte access
+template <typename T, int V> struct VecIO;
+template <> struct VecIO<bf16_t, 8> {
+  __device__ static __forceinline__ void ld(const bf16_t* p, float* o) {
+    const u16x8 a = *reinterpret_cast<const u16x8*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[2 * i] = bf16lo(a.w[i]), o[2 * i + 1] = bf16hi(a.w[i]);
+  }
+  __device__ static __forceinline__ void st(bf16_t* p, const float* v) {
+    u16x8 a;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a.w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
+    *reinterpret_cast<u16x8*>(p) = a;
+  }
+};
+template <> struct VecIO<float, 4> {
+  __device__ static __forceinline__ void ld(const float* p, float* o) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+    o[0] = a[0], o[1] = a[1], o[2] = a[2], o[3] = a[3];
+  }
+  __device__ static __forceinline__ void st(float* p, const float* v) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  }
+};
+template <typename T> struct VecIO<T, 1> {
+  __device__ static __forceinline__ void ld(const T* p, float* o) { o[0] = ldf<T>(p, 0); }
+  __device__ static __forceinline__ void st(T* p, const float* v) { stf<T>(p, 0, v[0]); }
+};
+
 struct LatentArgs {
   void* q_out;      // [T, H, r + dr]
   const void* qa;   // [H, T, r]: unrotated query parts times the key up-projection
@@ -44,8 +73,8 @@ struct LatentArgs {
   int T, H, r, dr;
 };
 
-// VEC: elements per 16-byte chunk when r, dr, the row strides and the bases allow whole chunks
-// (the query parts, the bulk of the bytes, are then copied chunk by chunk), else 1
+// VEC: elements per 16-byte chunk when r, dr, the rotated half, the row strides and the bases allow
+// whole chunks (the query rows, the bulk of the bytes, are then built chunk by chunk), else 1
 template <typename T, int VEC>
 __global__ void __launch_bounds__(256) latent_rope_kernel(LatentArgs g) {
   extern __shared__ float cs_sn[];  // [half] cosines, [half] sines, both times mag
@@ -84,17 +113,33 @@ __global__ void __launch_bounds__(256) latent_rope_kernel(LatentArgs g) {
   const T* q = (const T*)g.q + t * g.q_stride;
   T* qo = (T*)g.q_out + t * (int64_t)g.H * Wc;
   if constexpr (VEC > 1) {
+    // work items of VEC columns per head: copies of qa, rotated pairs of runs (a run of the low half
+    // with its partner of the high half, every angle used once), runs that are not rotated
     typedef uint32_t raw4 __attribute__((ext_vector_type(4)));
-    const int per = Wc / VEC;
+    const int n_copy = g.r / VEC, n_pair = g.half / VEC, per = n_copy + n_pair + (g.dr - 2 * g.half) / VEC;
     for (int it = tid; it < g.H * per; it += blockDim.x) {
-      const int h = it / per, c = (it - h * per) * VEC;
-      if (c < g.r) {
-        *reinterpret_cast<raw4*>(qo + (int64_t)h * Wc + c) =
-            *reinterpret_cast<const raw4*>((const T*)g.qa + ((int64_t)h * g.T + t) * g.r + c);
-      } else {
+      const int h = it / per, j = it - h * per;
+      T* dst = qo + (int64_t)h * Wc;
+      const T* src = q + (int64_t)h * g.q_head + g.q_off;
+      if (j < n_copy) {
+        *reinterpret_cast<raw4*>(dst + j * VEC) =
+            *reinterpret_cast<const raw4*>((const T*)g.qa + ((int64_t)h * g.T + t) * g.r + j * VEC);
+      } else if (j < n_copy + n_pair) {
+        const int e0 = (j - n_copy) * VEC;
+        float x[VEC], y[VEC], lo[VEC], hi[VEC];
+        VecIO<T, VEC>::ld(src + e0, x);
+        VecIO<T, VEC>::ld(src + g.half + e0, y);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-          stf<T>(qo, (int64_t)h * Wc + c + e, rot(q + (int64_t)h * g.q_head + g.q_off, c - g.r + e));
+        for (int e = 0; e < VEC; ++e) {
+          const float cs = cs_sn[e0 + e], sn = cs_sn[g.half + e0 + e];
+          lo[e] = x[e] * cs - y[e] * sn;
+          hi[e] = y[e] * cs + x[e] * sn;
+        }
+        VecIO<T, VEC>::st(dst + g.r + e0, lo);
+        VecIO<T, VEC>::st(dst + g.r + g.half + e0, hi);
+      } else {
+        const int e0 = 2 * g.half + (j - n_copy - n_pair) * VEC;
+        *reinterpret_cast<raw4*>(dst + g.r + e0) = *reinterpret_cast<const raw4*>(src + e0);
       }
     }
   } else {
@@ -120,7 +165,8 @@ extern "C" int dxm_latent_rope(void* q_out, const void* qa, const void* q, int64
                pos, slots, cache, T_, H, r, dr};
   const size_t lds = (size_t)2 * half * sizeof(float);
   const int V = f32 ? 4 : 8;
-  const bool vec = r % V == 0 && dr % V == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)qa % 16 == 0;
+  const bool vec = r % V == 0 && dr % V == 0 && half % V == 0 && q_stride % V == 0 && q_head % V == 0 && q_off % V == 0 &&
+                   (uintptr_t)q_out % 16 == 0 && (uintptr_t)qa % 16 == 0 && (uintptr_t)q % 16 == 0;
   if (f32 && vec) hipLaunchKernelGGL((latent_rope_kernel<float, 4>), dim3(T_), dim3(256), lds, st, g);
   else if (f32) hipLaunchKernelGGL((latent_rope_kernel<float, 1>), dim3(T_), dim3(256), lds, st, g);
   else if (vec) hipLaunchKernelGGL((latent_rope_kernel<bf16_t, 8>), dim3(T_), dim3(256), lds, st, g);

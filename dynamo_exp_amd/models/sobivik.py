@@ -335,7 +335,10 @@ class SobivikForCausalLM:
                 freq, mag = rc.yarn_frequencies(int(rot["dims"]), float(rot["base"]), rot.get("scaling")) \
                     if rot and rot.get("dims") else (None, 1.0)
                 sink = sd.get(p + "sink")
+                if sd[p + "dkv"].shape[0] != r + m["rot_dim"] or sd[p + "uq"].shape[0] != H * (d + m["rot_dim"]):
+                    raise ValueError(f"{p}: projection rows do not fit kv_rank, rot_dim, heads and dim")
                 out.update(w_in=act(p + "dq", p + "dkv", p + "g"), qn=f32(sd[p + "dq.norm"]), w_uq=act(p + "uq"),
+                           qr=int(sd[p + "dq"].shape[0]),  # the query latent's width is the tensor's
                            cn=f32(sd[p + "dkv.norm"]), sink=f32(sink) if sink is not None else None,
                            uk=sd[p + "uk"].to(dev, dt).view(H, d, r).contiguous(),
                            uv=sd[p + "uv"].to(dev, dt).view(H, dv, r).transpose(1, 2).contiguous(),
@@ -402,7 +405,7 @@ class SobivikForCausalLM:
 
     def _latent_attention(self, L: dict, h: torch.Tensor, meta: AttnMeta, cache, seq, tables, bs: int):
         m, T = L["m"], h.shape[0]
-        H, d, dr, dv, r, qr = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+        H, d, dr, dv, r, qr = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], L["qr"]
         eps = self.cfg.rms_norm_eps
         p = self._mm(h, L["w_in"])  # [query latent (q_rank) | key/value latent (kv_rank) | key part (rot_dim) | g]
         q = self._mm(mx.section_norm(p[:, :qr], L["qn"], eps), L["w_uq"])  # per head [dim unrotated | rot_dim]

@@ -1,7 +1,8 @@
 """Ops with per-sequence state: the generalized delta rule (a running matrix
-per head), retention (a running matrix with a fixed decay per head), short causal convolutions over time fused with rotary positions and
-the paged cache write, and the per-head unit-RMS + gate that follows a
-recurrent mixer.
+per head), retention (a running matrix with a fixed decay per head), short
+causal convolutions over time fused with rotary positions and the paged cache
+write, the query / key preparation of latent attention with a rotated key
+part, and the per-head unit-RMS + gate that follows a recurrent mixer.
 
 State lives in slots: state tensors are [slots, ...], the engine's KV manager
 hands a slot to every live request, and a step names the slot of each of its

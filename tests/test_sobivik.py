@@ -679,6 +679,45 @@ def test_greedy_generation(device, dtype, graphs):
             seq.append(t)
 
 
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_trace_replay_command(tmp_path, monkeypatch, capsys, device, dtype):
+    """The replay command on a checkpoint directory: the class follows config.json, a portion beside
+    a shorter one, a decode token beside a portion, a step in which nothing is wanted, a slot and
+    pages used again; logits files against the oracle."""
+    import io
+    import json
+    import sys
+
+    import numpy as np
+    from safetensors.torch import save_file
+
+    from dynamo_exp_amd.cli import trace_run
+
+    cfg = CONFIGS["mixed"]()
+    sd = weights(cfg, 21)
+    model_dir, out = tmp_path / "m", tmp_path / "out"
+    cfg.write_hf_config(str(model_dir))
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(model_dir / "model.safetensors"))
+    a, b = tokens(40, cfg.vocab_size, 31), tokens(9, cfg.vocab_size, 32)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:25], "want": [0, 24]},
+                                     {"id": "b", "tokens": b[:2], "want": [1]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[25:26], "want": [0]},
+                                     {"id": "b", "tokens": b[2:], "want": [0, 6]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[26:], "want": []}], "end": ["a"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": b, "want": [8]}], "end": ["c"]}]
+    monkeypatch.setattr(sys, "stdin", io.StringIO("\n".join(json.dumps(st) for st in steps) + "\n"))
+    rc_ = trace_run.main(["--model", str(model_dir), "--dtype", dtype, "--out", str(out), "--max-tokens", "128",
+                          "--device", device])
+    assert rc_ == 0
+    assert [ln for ln in capsys.readouterr().out.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    assert not (out / "2.f32").exists()
+    wa, wb = O.forward(cfg_dict(cfg), sd, a)[0], O.forward(cfg_dict(cfg), sd, b)[0]
+    got = {i: torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg.vocab_size)) for i in (0, 1, 3)}
+    close(got[0], torch.cat([wa[[0, 24]], wb[[1]]]), dtype, "step 0")
+    close(got[1], torch.cat([wa[[25]], wb[[2, 8]]]), dtype, "step 1")
+    close(got[3], wb[[8]], dtype, "step 3")
+
+
 def test_config_round_trip(tmp_path):
     """config.json keys -> LayeredConfig -> config.json; the preset builds and counts its weights."""
     cfg = CONFIGS["mixed"]()
@@ -689,3 +728,10 @@ def test_config_round_trip(tmp_path):
     tiny = get_config("sobivik-tiny")
     sd = SobivikForCausalLM(tiny, "cpu", torch.float32).random_state(0)
     assert sum(v.numel() for v in sd.values()) == tiny.num_params()
+    from dynamo_exp_amd.models.registry import build_model, supports_dtype
+
+    assert supports_dtype("Sobivik", "float32") and supports_dtype("Sobivik", "bfloat16")
+    assert isinstance(build_model(back, "cpu", dtype="float32"), SobivikForCausalLM)
+    with pytest.raises(ValueError):
+        SobivikForCausalLM(config([{"type": "general_delta", "mixer": {"heads": 1, "dim": 8}, "mlp": None}]), "cpu",
+                           torch.float32)
