@@ -651,7 +651,7 @@ extern "C" {
 
 // 1 when tile_attention has an instance for the head widths
 int dxm_tile_attention_ok(int d, int dv) {
-  const int pairs[][2] = {{2, 2}, {2, 4}, {3, 3}, {3, 6}, {4, 4}, {4, 8}, {8, 8}, {8, 16}, {9, 8}, {16, 12}, {16, 16}};
+  const int pairs[][2] = {{2, 2}, {2, 4}, {3, 3}, {3, 6}, {4, 4}, {4, 8}, {8, 8}, {8, 16}, {16, 12}, {16, 16}};
   for (auto& p : pairs)
     if (d == p[0] * 16 && dv == p[1] * 16) return 1;
   return 0;
@@ -678,7 +678,6 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
   TILE_CASE(4, 8)
   TILE_CASE(8, 8)
   TILE_CASE(8, 16)
-  TILE_CASE(9, 8)
   TILE_CASE(16, 12)
   TILE_CASE(16, 16)
   return 2;
@@ -708,7 +707,6 @@ int dxm_group_decode(float* ws, const void* q, int64_t q_stride, const void* kc,
   GROUP_CASE(4, 8)
   GROUP_CASE(8, 8)
   GROUP_CASE(8, 16)
-  GROUP_CASE(9, 8)
   GROUP_CASE(16, 12)
   GROUP_CASE(16, 16)
   return 2;

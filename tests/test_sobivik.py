@@ -425,7 +425,7 @@ def test_row_attention_keep_and_sink(device, size, keep, dims):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("size,keep", [(0, 0), (1, 1), (40, 7), (129, 70), (64, 64), (20, 200)])
-@pytest.mark.parametrize("dims", [(4, 2, 32, 32, 1), (4, 1, 32, 64, 2), (4, 1, 64, 128, 2), (3, 1, 144, 128, 1),
+@pytest.mark.parametrize("dims", [(4, 2, 32, 32, 1), (4, 1, 32, 64, 2), (4, 1, 64, 128, 2), (3, 1, 256, 192, 1),
                                   (20, 1, 256, 192, 1), (2, 2, 128, 128, 1)])
 def test_matrix_core_attention_keep_and_sink(size, keep, dims):
     """The matrix-core kernels with kept first keys and a sink: a 263-row portion that starts at
