@@ -37,6 +37,8 @@ namespace {
 constexpr int kRows = 128;  // rows per workgroup
 constexpr int kKeys = 64;   // keys per tile
 constexpr int kVtStride = kKeys + 8;
+// decode rows of wide heads: a narrower pad lets a third one-wave workgroup share a CU's LDS
+constexpr int kVtStrideWide = kKeys + 4;
 
 struct TileArgs {
   const bf16_t* q;
@@ -87,7 +89,7 @@ __device__ __forceinline__ int first_visible(int p, int mask, int size) {
 // are 16-byte chunks, consecutive threads on consecutive chunks of a row.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <int d, int dv, int NT>
+template <int d, int dv, int NT, int VS = kVtStride>
 struct TileStage {
   static constexpr int ks_stride = d + 8;
   static constexpr int kItems = kKeys * (d / 8), vItems = (kKeys / 4) * (dv / 8);
@@ -156,8 +158,8 @@ struct TileStage {
         lo.y = (vr[i][2][w] & 0xffffu) | (vr[i][3][w] << 16);
         hi2.x = (vr[i][0][w] >> 16) | (vr[i][1][w] & 0xffff0000u);
         hi2.y = (vr[i][2][w] >> 16) | (vr[i][3][w] & 0xffff0000u);
-        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w) * kVtStride + 4 * kg) = lo;
-        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w + 1) * kVtStride + 4 * kg) = hi2;
+        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w) * VS + 4 * kg) = lo;
+        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w + 1) * VS + 4 * kg) = hi2;
       }
     }
   }
@@ -495,7 +497,8 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   // wide heads: a whole tile in flight would not fit the register file beside the
   // accumulators, so K and V are staged one after the other and nothing is prefetched
   constexpr bool kWide = DB + DVB > 16;
-  TileStage<d, dv, 64> stage;
+  constexpr int VS = kWide ? kVtStrideWide : kVtStride;
+  TileStage<d, dv, 64, VS> stage;
   if (!kWide && t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, t0 * kKeys, nf, shift, p, lane);
   for (int t = t0; t < t1; ++t) {
     const int ut = t * kKeys;
@@ -567,7 +570,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
       for (int cb = 0; cb < DVB; ++cb) {
-        const i16x4 A = *reinterpret_cast<const i16x4*>(Vt + (cb * 16 + c16) * kVtStride + kb * 16 + 4 * g4);
+        const i16x4 A = *reinterpret_cast<const i16x4*>(Vt + (cb * 16 + c16) * VS + kb * 16 + 4 * g4);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
           O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Ph[qb][kb], O[qb][cb], 0, 0, 0);
@@ -596,7 +599,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
 
 template <int DB, int DVB>
 int launch_group(const GroupArgs& a0, int rows, hipStream_t st) {
-  const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * kVtStride) * sizeof(bf16_t);
+  const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * (DB + DVB > 16 ? kVtStrideWide : kVtStride)) * sizeof(bf16_t);
   GroupArgs a = a0;
   const bool two = a.group > 16 && DB + DVB <= 16;  // two head blocks per wave only where the registers hold them
   a.chunks = two ? (a.group + 31) / 32 : (a.group + 15) / 16;
